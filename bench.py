@@ -1,0 +1,232 @@
+"""Benchmark of the MoE expert-layer forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3] [--no-cpu-baseline]
+
+A step is one whole-layer forward (router -> dispatch -> grouped SwiGLU ->
+shared experts -> combine) over one batch of synthetic, seeded input that is
+already resident in HBM.  The timed region is exactly K calls of the C entry
+point jtmoe_moe_forward bracketed by torch.cuda.synchronize().  After it, K more
+steps are run through jtmoe_moe_forward_timed, which records a hipEvent on the
+launch stream after every stage; the per-stage averages give the roofline
+figures.  Prints ONE JSON line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3
+
+
+def algorithmic_work(cfg: dict) -> dict:
+    """Algorithmic flops / bytes per launch of each stage (one unit = one layer call)."""
+    T = cfg["batch"] * cfg["seq"]
+    H, E, K, I, Ns = cfg["H"], cfg["E"], cfg["K"], cfg["I"], cfg["Ns"]
+    b = 2 if cfg["dtype"] == "bf16" else 4
+    A = T * K
+    Is = I * Ns
+    return dict(
+        router_bytes=T * H * b + H * E * b + E * 4 + A * 4 + A * b + T * E * 4,
+        dispatch_bytes=A * 4 + 2 * E * 4 + 2 * A * 4 + T * H * b + A * H * b,
+        dispatch_rows_bytes=A * 4 + T * H * b + A * H * b,
+        combine_bytes=A * H * b + A * b + A * 4 + T * H * b + (T * H * b if Ns else 0),
+        gate_up_flops=4 * A * H * I,
+        down_flops=2 * A * I * H,
+        shared_gate_up_flops=4 * T * H * Is,
+        shared_down_flops=2 * T * Is * H,
+        router_flops=2 * T * H * E,
+    )
+
+
+def cpu_baseline(name: str, sample_tokens: int) -> dict:
+    """The oracle (a NumPy port of the reference layer) timed on the host cores,
+    on the first `sample_tokens` tokens of the same seeded workload."""
+    import numpy as np
+
+    from oracle import moe_oracle as O
+
+    inp = O.make_inputs(name, seed=0, tokens=sample_tokens)
+    cfg = inp["cfg"]
+    kwargs = dict(top_k=cfg["K"], route_scale=1.0, dtype=cfg["dtype"], shared=inp["shared"])
+    args = (inp["x"], inp["w_router"], inp["expert_bias"], inp["gate"], inp["up"], inp["down"])
+    small = inp["x"][:, : min(64, sample_tokens)]
+    O.moe_forward(small, *args[1:], **kwargs)  # first call excluded
+    t0 = time.perf_counter()
+    out = O.moe_forward(*args, **kwargs)
+    dt = time.perf_counter() - t0
+    assert np.isfinite(out.y).all()
+    cores = len(os.sched_getaffinity(0))
+    try:
+        from threadpoolctl import threadpool_info
+
+        blas = [p.get("num_threads") for p in threadpool_info() if p.get("user_api") == "blas"]
+        if blas:
+            cores = int(max(blas))
+    except Exception:
+        pass
+    return dict(
+        value=sample_tokens / dt,
+        unit="tokens/s",
+        cores=cores,
+        kind="port",
+        sample=f"first {sample_tokens} tokens of {name} (same seed-0 weights), NumPy oracle with emulated "
+               f"{cfg['dtype']}, one timed call of {dt:.2f} s after a 64-token warm-up call",
+    )
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--config", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
+    parser.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: the layer runs with every expert local and no collective; "
+              f"--gpus {args.gpus} is not supported in this build", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from research_amd import _ffi, ops
+    from research_amd.synthetic import DESCRIPTIONS, make_inputs
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU path)", file=sys.stderr)
+        return 2
+    _ffi.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    inp = make_inputs(args.config, seed=0)
+    cfg = inp["cfg"]
+    tdtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    T = cfg["batch"] * cfg["seq"]
+
+    def up(a):
+        return torch.from_numpy(a).to(dev).to(tdtype).contiguous()
+
+    x = up(inp["x"].reshape(T, cfg["H"]))
+    w_r, gate, upw, down = up(inp["w_router"]), up(inp["gate"]), up(inp["up"]), up(inp["down"])
+    bias = torch.from_numpy(inp["expert_bias"]).to(dev)
+    shared = None if inp["shared"] is None else tuple(up(m) for m in inp["shared"])
+    del inp
+    torch.cuda.synchronize()
+
+    def step(stage_ms=None):
+        return ops.moe_forward(x, w_r, bias, gate, upw, down, cfg["K"], 1.0, shared=shared, stage_ms=stage_ms)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # per-call latencies (the reference's protocol: perf_counter around a blocking call)
+    lat = []
+    for _ in range(max(args.steps, 10)):
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        step()
+        torch.cuda.synchronize()
+        lat.append((time.perf_counter() - t1) * 1e3)
+    lat.sort()
+
+    # per-stage durations from hipEvents on the launch stream
+    per_stage = [[] for _ in range(_ffi.NUM_STAGES)]
+    for _ in range(args.steps):
+        ms: list = []
+        result = step(ms)
+        for i, v in enumerate(ms):
+            per_stage[i].append(v)
+    stage_ms = {name: (sum(v) / len(v) if v else 0.0) for name, v in zip(_ffi.STAGE_NAMES, per_stage)}
+    group_sizes = result.group_sizes.cpu().tolist()
+
+    work = algorithmic_work(cfg)
+    peak = MFMA_BF16_PEAK_TFLOPS if cfg["dtype"] == "bf16" else MFMA_F32_PEAK_TFLOPS
+
+    def tflops(flops, ms):
+        return flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+
+    def gbs(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+
+    gate_up_tf = tflops(work["gate_up_flops"], stage_ms["gate_up"])
+    roofline = dict(
+        kernel="grouped gate/up GEMM + SwiGLU (routed experts)",
+        bound="mfma",
+        achieved=gate_up_tf,
+        peak=peak,
+        unit="TFLOP/s",
+        frac=gate_up_tf / peak,
+        traffic=None,
+        avg_launch_ms=stage_ms["gate_up"],
+        flops_per_launch=work["gate_up_flops"],
+    )
+    dispatch_ms = stage_ms["dispatch_meta"] + stage_ms["dispatch_rows"]
+    stages = dict(
+        ms=stage_ms,
+        grouped_gemm_mfma_util=tflops(work["gate_up_flops"] + work["down_flops"], stage_ms["gate_up"] + stage_ms["down"]) / peak,
+        down_tflops=tflops(work["down_flops"], stage_ms["down"]),
+        shared_tflops=tflops(work["shared_gate_up_flops"] + work["shared_down_flops"],
+                             stage_ms["shared_gate_up"] + stage_ms["shared_down"]),
+        router_gbs=gbs(work["router_bytes"], stage_ms["router"]),
+        dispatch_gbs=gbs(work["dispatch_bytes"], dispatch_ms),
+        dispatch_rows_gbs=gbs(work["dispatch_rows_bytes"], stage_ms["dispatch_rows"]),
+        combine_gbs=gbs(work["combine_bytes"], stage_ms["combine"]),
+        hbm_peak_gbs=HBM_PEAK_GBS,
+    )
+
+    line = {
+        "metric": "MoE layer tokens/s (64E top-8, d2048); grouped-GEMM MFMA util %",
+        "value": T / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.config}: {DESCRIPTIONS[args.config]}; x~N(0,1), weights~N(0,0.02), seed 0, "
+                        "sigmoid top-k router (the reference's), inputs resident in HBM",
+            "tokens": T, "d_model": cfg["H"], "experts": cfg["E"], "top_k": cfg["K"], "d_ff": cfg["I"],
+            "shared_experts": cfg["Ns"],
+            "group_rows_min_max": [min(group_sizes), max(group_sizes)],
+        },
+        "latency_ms": {
+            "median": statistics.median(lat), "p10": lat[int(0.1 * (len(lat) - 1))],
+            "p90": lat[int(0.9 * (len(lat) - 1))], "min": lat[0], "max": lat[-1],
+        },
+        "roofline": roofline,
+        "stages": stages,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.config, min(args.cpu_sample_tokens, T))
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

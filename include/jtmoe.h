@@ -1,0 +1,212 @@
+/*
+ * jtmoe.h -- C ABI of libjtmoe.so: the MoE expert-layer forward of Jaxtitan
+ * (vpareek2/research, src/jaxtitan/models/components/moe.py) on AMD gfx950.
+ *
+ * Conventions (they follow the reference's native-kernel boundary,
+ * src/jaxtitan/kernels/cuda/rmsnorm/rmsnorm_ffi.cu:24-74):
+ *   - every pointer is a DEVICE pointer to a dense row-major array; the caller
+ *     owns every buffer, results and workspace are pre-allocated by the caller;
+ *   - a launcher validates its arguments, enqueues kernels on `stream` only and
+ *     returns; it never allocates, frees, synchronises or retains a pointer;
+ *   - return value 0 (JTMOE_OK) or a negative JTMOE_E* code; the message of the
+ *     last failure on the calling thread is `jtmoe_last_error()`;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - `dtype` selects the compute dtype of activations and weights:
+ *     JTMOE_BF16 (2-byte elements) or JTMOE_F32 (4-byte elements).
+ *
+ * Index conventions: T tokens, H hidden size, E experts, K = top_k,
+ * I = expert intermediate size, A = T*K assignments; assignment a = t*K + s
+ * (moe.py:583-586).
+ */
+#ifndef JTMOE_H_
+#define JTMOE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JTMOE_VERSION 1
+
+enum {
+  JTMOE_BF16 = 0,
+  JTMOE_F32 = 1
+};
+
+enum {
+  JTMOE_OK = 0,
+  JTMOE_EINVAL = -1,       /* bad pointer, shape or attribute                    */
+  JTMOE_EUNSUPPORTED = -2, /* valid request outside the implemented envelope     */
+  JTMOE_EWORKSPACE = -3,   /* workspace too small                                */
+  JTMOE_ELAUNCH = -4       /* hipGetLastError() after a launch reported an error */
+};
+
+/* Limits of the implementation. */
+#define JTMOE_MAX_EXPERTS 256
+#define JTMOE_MAX_TOP_K 16
+
+int jtmoe_version(void);
+
+/* Message of the last error returned on this thread ("" if none). */
+const char* jtmoe_last_error(void);
+
+/*
+ * Router.  Replaces SigmoidTopKRouter.__call__ (moe.py:131-147):
+ *   logits = f32(round_dtype(x @ w_router)); scores = sigmoid(logits);
+ *   ids = top_k(scores + expert_bias, K)  (descending; equal values -> lower index);
+ *   weights = scores[ids] / (sum_k scores[ids] + 1e-20) * route_scale, cast to dtype.
+ * and the two vectors of _router_stats (moe.py:802-805):
+ *   expert_counts[e] = #{(t,s): ids[t,s]==e},  importance[e] = sum of their weights.
+ *
+ *   x [T,H] dtype; w_router [H,E] dtype; expert_bias [E] f32 or NULL (= zeros).
+ *   out: expert_ids [T,K] i32; weights [T,K] dtype; scores [T,E] f32;
+ *        expert_counts [E] f32; importance [E] f32; logits [T,E] f32 or NULL.
+ *   workspace: jtmoe_router_workspace_bytes(E) bytes.
+ */
+size_t jtmoe_router_workspace_bytes(int64_t E);
+int jtmoe_router(const void* x, const void* w_router, const float* expert_bias,
+                 int64_t T, int64_t H, int64_t E, int64_t K, double route_scale, int dtype,
+                 int32_t* expert_ids, void* weights, float* scores,
+                 float* expert_counts, float* importance, float* logits,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The same router, starting from given fp32 logits [T,E] (moe.py:133-147 only).
+ * The routing decision is a pure function of the logits, identical bit for bit
+ * to what jtmoe_router derives from its own logits.
+ */
+int jtmoe_router_from_logits(const float* logits, const float* expert_bias,
+                             int64_t T, int64_t E, int64_t K, double route_scale, int dtype,
+                             int32_t* expert_ids, void* weights, float* scores,
+                             float* expert_counts, float* importance,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Token dispatch.  Replaces the single-device part of local_dispatch
+ * (moe.py:583-602): per-expert histogram, exclusive prefix sum, the stable
+ * permutation of assignments into expert-contiguous order and its inverse, and
+ * the row gather packed_x[j] = x[source_order[j] / K].
+ *
+ *   expert_ids [A] i32, each in [0,E) (duplicates within a token are legal);
+ *   x [T,H] dtype, or NULL to skip the row gather (then packed_x is ignored).
+ *   out: group_sizes [E] i32; offsets [E] i32; source_order [A] i32;
+ *        inverse [A] i32; packed_x [A,H] dtype.
+ *   workspace: jtmoe_dispatch_workspace_bytes(T*K, E) bytes.
+ * An id outside [0,E) is not detected on the host (ids live on the device); such
+ * an assignment is dropped from the permutation.
+ */
+size_t jtmoe_dispatch_workspace_bytes(int64_t A, int64_t E);
+int jtmoe_dispatch(const int32_t* expert_ids, const void* x,
+                   int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
+                   int32_t* group_sizes, int32_t* offsets,
+                   int32_t* source_order, int32_t* inverse, void* packed_x,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Grouped SwiGLU expert FFN.  Replaces the three jax.lax.ragged_dot calls and
+ * the SwiGLU between them (moe.py:638-641):
+ *   rows offsets[e] .. offsets[e]+group_sizes[e]-1 of packed_x use expert e;
+ *   act = silu(packed_x @ gate[e]) * (packed_x @ up[e]);  packed_y = act @ down[e].
+ *
+ *   packed_x [A,H] dtype; gate, up [E,H,I] dtype; down [E,I,H] dtype;
+ *   group_sizes, offsets [E] i32 (device); act [A,I] dtype (workspace, overwritten);
+ *   out: packed_y [A,H] dtype.  Groups of size 0 cost nothing.
+ */
+int jtmoe_grouped_swiglu(const void* packed_x, const void* gate, const void* up, const void* down,
+                         const int32_t* group_sizes, const int32_t* offsets,
+                         int64_t A, int64_t H, int64_t I, int64_t E, int dtype,
+                         void* act, void* packed_y, void* stream);
+
+/*
+ * Shared experts.  Replaces SharedSwiGLU.__call__ (moe.py:361-364) on one device
+ * (execution.py:186-187, 199-200): one dense SwiGLU of width Is = I*num_shared.
+ *   x [T,H]; gate, up [H,Is]; down [Is,H]; act [T,Is] workspace; out shared_y [T,H].
+ */
+int jtmoe_shared_swiglu(const void* x, const void* gate, const void* up, const void* down,
+                        int64_t T, int64_t H, int64_t Is, int dtype,
+                        void* act, void* shared_y, void* stream);
+
+/*
+ * Combine.  Replaces the unpermute / weight / reduce of moe.py:663-671 and the
+ * unweighted shared-expert add of moe.py:415, 429:
+ *   y[t] = round_dtype( sum_s round_dtype(packed_y[inverse[t*K+s]] * weights[t,s]) )
+ *   (fp32 accumulation in slot order), then y[t] = round_dtype(y[t] + shared_y[t]).
+ *   packed_y [A,H]; inverse [A] i32; weights [T,K] dtype; shared_y [T,H] or NULL.
+ */
+int jtmoe_combine(const void* packed_y, const int32_t* inverse, const void* weights,
+                  const void* shared_y, int64_t T, int64_t H, int64_t K, int dtype,
+                  void* y, void* stream);
+
+/*
+ * Scalar router statistics.  Replaces the scalar fields of _router_stats
+ * (moe.py:806-813) derived from expert_counts [E] f32:
+ *   stats6 = {total_assignments, load_min, load_max, load_mean, max_vio, load_entropy}
+ *   max_vio = (load_max - mean) / max(mean, 1e-6);  entropy = -sum_{p>0} p ln p, p = counts / max(total, 1e-6).
+ */
+int jtmoe_router_stats(const float* expert_counts, int64_t E, float* stats6, void* stream);
+
+/*
+ * Sequence balance loss.  Replaces _sequence_balance_loss (moe.py:828-840):
+ *   f[b,e] = E/(K*S) * #{(s,k): ids[b,s,k]==e};  p[b,e] = mean_s scores[b,s,e]/max(sum_e scores, 1e-20);
+ *   loss = sum_{b,e} f*p / B.
+ *   expert_ids [B,S,K] i32; scores [B,S,E] f32; out loss [1] f32.
+ *   workspace: jtmoe_balance_workspace_bytes(B, E) bytes.
+ */
+size_t jtmoe_balance_workspace_bytes(int64_t B, int64_t E);
+int jtmoe_sequence_balance_loss(const int32_t* expert_ids, const float* scores,
+                                int64_t B, int64_t S, int64_t E, int64_t K,
+                                float* loss, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The whole layer.  Replaces SparseMoE.__call__ / forward_with_output
+ * (moe.py:411-446): router -> dispatch -> grouped SwiGLU -> (shared experts) ->
+ * combine, enqueued back to back on `stream`.
+ *
+ *   shared_gate/up [H,Is], shared_down [Is,H], or all NULL with Is == 0.
+ *   out: y [T,H]; expert_ids [T,K]; weights [T,K]; scores [T,E];
+ *        expert_counts, importance [E] f32; group_sizes, offsets [E] i32;
+ *        source_order, inverse [A] i32.
+ *   workspace: jtmoe_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype);
+int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_bias,
+                      const void* gate, const void* up, const void* down,
+                      const void* shared_gate, const void* shared_up, const void* shared_down,
+                      int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                      double route_scale, int dtype,
+                      void* y, int32_t* expert_ids, void* weights, float* scores,
+                      float* expert_counts, float* importance,
+                      int32_t* group_sizes, int32_t* offsets,
+                      int32_t* source_order, int32_t* inverse,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Measurement aid with no counterpart in the reference (its benchmarks time
+ * whole calls, src/jaxtitan/runtime/profile_bench.py:232-270): one
+ * jtmoe_moe_forward with a hipEvent recorded on `stream` after every stage.
+ * Unlike every other entry point it creates events and SYNCHRONISES the stream.
+ * stage_ms is a HOST array of JTMOE_NUM_STAGES floats, milliseconds per stage:
+ *   {router, dispatch (histogram+scan+rank), dispatch (row scatter),
+ *    routed gate/up GEMM + SwiGLU, routed down GEMM,
+ *    shared gate/up GEMM + SwiGLU, shared down GEMM, combine}.
+ */
+#define JTMOE_NUM_STAGES 8
+int jtmoe_moe_forward_timed(const void* x, const void* w_router, const float* expert_bias,
+                            const void* gate, const void* up, const void* down,
+                            const void* shared_gate, const void* shared_up, const void* shared_down,
+                            int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                            double route_scale, int dtype,
+                            void* y, int32_t* expert_ids, void* weights, float* scores,
+                            float* expert_counts, float* importance,
+                            int32_t* group_sizes, int32_t* offsets,
+                            int32_t* source_order, int32_t* inverse,
+                            void* workspace, size_t workspace_bytes, void* stream,
+                            float* stage_ms);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* JTMOE_H_ */

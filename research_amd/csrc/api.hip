@@ -1,0 +1,330 @@
+// Library-level pieces of libjtmoe: error state, the sequence balance loss and
+// the whole-layer launcher that chains the stage launchers on one stream.
+#include "common.hpp"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace jtmoe {
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void clear_error() { g_error[0] = '\0'; }
+
+thread_local StageTimer* g_stage_timer = nullptr;
+
+int check_launch(const char* what) {
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return fail(JTMOE_ELAUNCH, "%s: %s", what, hipGetErrorString(err));
+  return JTMOE_OK;
+}
+
+namespace {
+
+// ---- sequence balance loss (reference moe.py:828-840) --------------------------
+constexpr int kBalThreads = 256;
+constexpr int kBalWaves = kBalThreads / kWave;
+constexpr int kBalPerLane = JTMOE_MAX_EXPERTS / kWave;
+
+__global__ __launch_bounds__(kBalThreads) void balance_partial_kernel(const int32_t* __restrict__ ids,
+                                                                      const float* __restrict__ scores, int S, int E,
+                                                                      int K, float* __restrict__ partial) {
+  extern __shared__ float smem[];
+  float* psum = smem;                                        // [kBalWaves][E]
+  int* cnt = reinterpret_cast<int*>(smem + kBalWaves * E);   // [E]
+  __shared__ float red[kBalWaves];
+  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int e = tid; e < E; e += kBalThreads) cnt[e] = 0;
+  __syncthreads();
+  const int32_t* ids_b = ids + (size_t)b * S * K;
+  for (int i = tid; i < S * K; i += kBalThreads) {
+    const int id = ids_b[i];
+    if (id >= 0 && id < E) atomicAdd(&cnt[id], 1);
+  }
+  float acc[kBalPerLane];
+#pragma unroll
+  for (int j = 0; j < kBalPerLane; ++j) acc[j] = 0.0f;
+  for (int s = wave; s < S; s += kBalWaves) {
+    const float* row = scores + ((size_t)b * S + s) * E;
+    float v[kBalPerLane];
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kBalPerLane; ++j) {
+      const int e = lane + j * kWave;
+      v[j] = e < E ? row[e] : 0.0f;
+      sum += v[j];
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
+    const float d = fmaxf(sum, 1e-20f);
+#pragma unroll
+    for (int j = 0; j < kBalPerLane; ++j) acc[j] += v[j] / d;
+  }
+#pragma unroll
+  for (int j = 0; j < kBalPerLane; ++j) {
+    const int e = lane + j * kWave;
+    if (e < E) psum[wave * E + e] = acc[j];
+  }
+  __syncthreads();
+  const float fscale = (float)E / ((float)K * (float)S);
+  float local = 0.0f;
+  for (int e = tid; e < E; e += kBalThreads) {
+    float p = 0.0f;
+    for (int w = 0; w < kBalWaves; ++w) p += psum[w * E + e];
+    p = p / (float)S;
+    local += fscale * (float)cnt[e] * p;
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) local += __shfl_xor(local, m);
+  if (lane == 0) red[wave] = local;
+  __syncthreads();
+  if (tid == 0) {
+    float t = 0.0f;
+    for (int w = 0; w < kBalWaves; ++w) t += red[w];
+    partial[b] = t;
+  }
+}
+
+__global__ void balance_final_kernel(const float* __restrict__ partial, int B, float* __restrict__ loss) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    float t = 0.0f;
+    for (int b = 0; b < B; ++b) t += partial[b];
+    loss[0] = t / (float)B;
+  }
+}
+
+// ---- scalar router statistics (reference moe.py:806-813) -----------------------
+// out = {total, load_min, load_max, load_mean, max_vio, load_entropy}
+__global__ __launch_bounds__(256) void router_stats_kernel(const float* __restrict__ counts, int E,
+                                                           float* __restrict__ out) {
+  __shared__ float s_sum[256], s_min[256], s_max[256];
+  const int tid = threadIdx.x;
+  float sum = 0.0f, mn = 3.402823466e38f, mx = -3.402823466e38f;
+  for (int e = tid; e < E; e += 256) {
+    const float c = counts[e];
+    sum += c;
+    mn = fminf(mn, c);
+    mx = fmaxf(mx, c);
+  }
+  s_sum[tid] = sum;
+  s_min[tid] = mn;
+  s_max[tid] = mx;
+  __syncthreads();
+  for (int d = 128; d >= 1; d >>= 1) {
+    if (tid < d) {
+      s_sum[tid] += s_sum[tid + d];
+      s_min[tid] = fminf(s_min[tid], s_min[tid + d]);
+      s_max[tid] = fmaxf(s_max[tid], s_max[tid + d]);
+    }
+    __syncthreads();
+  }
+  const float total = s_sum[0];
+  const float lmin = s_min[0], lmax = s_max[0];
+  __syncthreads();
+  float ent = 0.0f;
+  const float denom = fmaxf(total, 1e-6f);
+  for (int e = tid; e < E; e += 256) {
+    const float p = counts[e] / denom;
+    if (p > 0.0f) ent += p * logf(p);
+  }
+  s_sum[tid] = ent;
+  __syncthreads();
+  for (int d = 128; d >= 1; d >>= 1) {
+    if (tid < d) s_sum[tid] += s_sum[tid + d];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    const float mean = total / (float)E;
+    out[0] = total;
+    out[1] = lmin;
+    out[2] = lmax;
+    out[3] = mean;
+    out[4] = (lmax - mean) / fmaxf(mean, 1e-6f);
+    out[5] = -s_sum[0];
+  }
+}
+
+struct Carve {
+  unsigned char* base;
+  size_t used;
+  void* take(size_t bytes) {
+    void* p = base ? base + used : nullptr;
+    used += align_up(bytes, 256);
+    return p;
+  }
+};
+
+struct LayerWorkspace {
+  void* router;
+  size_t router_bytes;
+  void* dispatch;
+  size_t dispatch_bytes;
+  void* packed_x;
+  void* act;
+  void* packed_y;
+  void* shared_act;
+  void* shared_y;
+  size_t total;
+};
+
+LayerWorkspace carve_layer(void* base, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype) {
+  const size_t b = dtype_bytes(dtype);
+  const size_t A = (size_t)T * (size_t)K;
+  Carve c{static_cast<unsigned char*>(base), 0};
+  LayerWorkspace w;
+  w.router_bytes = jtmoe_router_workspace_bytes(E);
+  w.router = c.take(w.router_bytes);
+  w.dispatch_bytes = jtmoe_dispatch_workspace_bytes((int64_t)A, E);
+  w.dispatch = c.take(w.dispatch_bytes);
+  w.packed_x = c.take(A * (size_t)H * b);
+  w.act = c.take(A * (size_t)I * b);
+  w.packed_y = c.take(A * (size_t)H * b);
+  w.shared_act = Is > 0 ? c.take((size_t)T * (size_t)Is * b) : nullptr;
+  w.shared_y = Is > 0 ? c.take((size_t)T * (size_t)H * b) : nullptr;
+  w.total = c.used;
+  return w;
+}
+
+}  // namespace
+}  // namespace jtmoe
+
+using namespace jtmoe;
+
+extern "C" int jtmoe_version(void) { return JTMOE_VERSION; }
+
+extern "C" const char* jtmoe_last_error(void) { return g_error; }
+
+extern "C" size_t jtmoe_balance_workspace_bytes(int64_t B, int64_t E) {
+  (void)E;
+  if (B <= 0) return 0;
+  return align_up((size_t)B * sizeof(float), 256);
+}
+
+extern "C" int jtmoe_sequence_balance_loss(const int32_t* expert_ids, const float* scores, int64_t B, int64_t S,
+                                           int64_t E, int64_t K, float* loss, void* workspace,
+                                           size_t workspace_bytes, void* stream) {
+  clear_error();
+  JT_REQUIRE(B > 0 && S > 0 && E > 0 && K > 0, "sequence_balance_loss: B=%lld S=%lld E=%lld K=%lld out of range",
+             (long long)B, (long long)S, (long long)E, (long long)K);
+  if (E > JTMOE_MAX_EXPERTS) return fail(JTMOE_EUNSUPPORTED, "sequence_balance_loss: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  JT_REQUIRE(B * S * E < ((int64_t)1 << 40) && S * K < ((int64_t)1 << 31) && B < ((int64_t)1 << 24),
+             "sequence_balance_loss: sizes out of range");
+  JT_REQUIRE(expert_ids && scores && loss && workspace, "sequence_balance_loss: null pointer argument");
+  if (workspace_bytes < jtmoe_balance_workspace_bytes(B, E))
+    return fail(JTMOE_EWORKSPACE, "sequence_balance_loss: workspace %zu < %zu bytes", workspace_bytes,
+                jtmoe_balance_workspace_bytes(B, E));
+  hipStream_t s = as_stream(stream);
+  float* partial = static_cast<float*>(workspace);
+  const size_t smem = (size_t)(kBalWaves + 1) * E * sizeof(float);
+  balance_partial_kernel<<<(unsigned)B, kBalThreads, smem, s>>>(expert_ids, scores, (int)S, (int)E, (int)K, partial);
+  balance_final_kernel<<<1, 64, 0, s>>>(partial, (int)B, loss);
+  return check_launch("sequence_balance_loss");
+}
+
+extern "C" int jtmoe_router_stats(const float* expert_counts, int64_t E, float* stats6, void* stream) {
+  clear_error();
+  JT_REQUIRE(E > 0 && E < ((int64_t)1 << 24), "router_stats: E=%lld out of range", (long long)E);
+  JT_REQUIRE(expert_counts && stats6, "router_stats: null pointer argument");
+  router_stats_kernel<<<1, 256, 0, as_stream(stream)>>>(expert_counts, (int)E, stats6);
+  return check_launch("router_stats");
+}
+
+extern "C" size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                                        int dtype) {
+  if (T < 0 || H <= 0 || E <= 0 || K <= 0 || I <= 0 || Is < 0 || !dtype_ok(dtype)) return 0;
+  return carve_layer(nullptr, T, H, E, K, I, Is, dtype).total;
+}
+
+extern "C" int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_bias, const void* gate,
+                                 const void* up, const void* down, const void* shared_gate, const void* shared_up,
+                                 const void* shared_down, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I,
+                                 int64_t Is, double route_scale, int dtype, void* y, int32_t* expert_ids,
+                                 void* weights, float* scores, float* expert_counts, float* importance,
+                                 int32_t* group_sizes, int32_t* offsets, int32_t* source_order, int32_t* inverse,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  JT_REQUIRE(dtype_ok(dtype), "moe_forward: unknown dtype %d", dtype);
+  JT_REQUIRE(T >= 0 && H > 0 && E > 0 && K > 0 && I > 0 && Is >= 0, "moe_forward: shape out of range");
+  JT_REQUIRE((Is == 0) == (shared_gate == nullptr) && (Is == 0) == (shared_up == nullptr) &&
+                 (Is == 0) == (shared_down == nullptr),
+             "moe_forward: shared expert matrices and Is=%lld disagree", (long long)Is);
+  JT_REQUIRE(workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
+             "moe_forward: workspace must be non-null and 256-byte aligned");
+  const LayerWorkspace w = carve_layer(workspace, T, H, E, K, I, Is, dtype);
+  if (workspace_bytes < w.total)
+    return fail(JTMOE_EWORKSPACE, "moe_forward: workspace %zu < %zu bytes", workspace_bytes, w.total);
+  int rc = jtmoe_router(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
+                        expert_counts, importance, nullptr, w.router, w.router_bytes, stream);
+  if (rc) return rc;
+  stage_mark(kStageRouter, as_stream(stream));
+  rc = jtmoe_dispatch(expert_ids, T > 0 ? x : nullptr, T, H, E, K, dtype, group_sizes, offsets, source_order,
+                      inverse, w.packed_x, w.dispatch, w.dispatch_bytes, stream);
+  if (rc) return rc;
+  rc = jtmoe_grouped_swiglu(w.packed_x, gate, up, down, group_sizes, offsets, T * K, H, I, E, dtype, w.act,
+                            w.packed_y, stream);
+  if (rc) return rc;
+  if (Is > 0) {
+    rc = jtmoe_shared_swiglu(x, shared_gate, shared_up, shared_down, T, H, Is, dtype, w.shared_act, w.shared_y,
+                             stream);
+    if (rc) return rc;
+  }
+  rc = jtmoe_combine(w.packed_y, inverse, weights, Is > 0 ? w.shared_y : nullptr, T, H, K, dtype, y, stream);
+  stage_mark(kStageCombine, as_stream(stream));
+  return rc;
+}
+
+extern "C" int jtmoe_moe_forward_timed(const void* x, const void* w_router, const float* expert_bias,
+                                       const void* gate, const void* up, const void* down, const void* shared_gate,
+                                       const void* shared_up, const void* shared_down, int64_t T, int64_t H,
+                                       int64_t E, int64_t K, int64_t I, int64_t Is, double route_scale, int dtype,
+                                       void* y, int32_t* expert_ids, void* weights, float* scores,
+                                       float* expert_counts, float* importance, int32_t* group_sizes,
+                                       int32_t* offsets, int32_t* source_order, int32_t* inverse, void* workspace,
+                                       size_t workspace_bytes, void* stream, float* stage_ms) {
+  clear_error();
+  JT_REQUIRE(stage_ms != nullptr, "moe_forward_timed: stage_ms is null");
+  StageTimer timer;
+  int created = 0;
+  for (; created < kStageCount; ++created)
+    if (hipEventCreate(&timer.ev[created]) != hipSuccess) break;
+  int rc = JTMOE_OK;
+  if (created != kStageCount) {
+    rc = fail(JTMOE_ELAUNCH, "moe_forward_timed: hipEventCreate failed");
+  } else {
+    hipStream_t s = as_stream(stream);
+    // every event is recorded once up front so that a skipped stage reads as zero
+    for (int i = kStageCount - 1; i >= 0; --i) (void)hipEventRecord(timer.ev[i], s);
+    g_stage_timer = &timer;
+    rc = jtmoe_moe_forward(x, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H, E, K,
+                           I, Is, route_scale, dtype, y, expert_ids, weights, scores, expert_counts, importance,
+                           group_sizes, offsets, source_order, inverse, workspace, workspace_bytes, stream);
+    g_stage_timer = nullptr;
+    if (hipStreamSynchronize(s) != hipSuccess && rc == JTMOE_OK)
+      rc = fail(JTMOE_ELAUNCH, "moe_forward_timed: stream synchronisation failed");
+    if (rc == JTMOE_OK) {
+      int last = kStageBegin;
+      for (int i = 1; i < kStageCount; ++i) {
+        float ms = 0.0f;
+        // a stage that did not run keeps its up-front record, which precedes kStageBegin
+        if (hipEventElapsedTime(&ms, timer.ev[last], timer.ev[i]) != hipSuccess || ms < 0.0f) {
+          stage_ms[i - 1] = 0.0f;
+          continue;
+        }
+        stage_ms[i - 1] = ms;
+        last = i;
+      }
+    }
+  }
+  for (int i = 0; i < created; ++i) (void)hipEventDestroy(timer.ev[i]);
+  return rc;
+}

@@ -1,0 +1,89 @@
+// Shared host/device helpers of libjtmoe (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "jtmoe.h"
+
+namespace jtmoe {
+
+// ---- host side: status + thread-local message -----------------------------
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+// hipGetLastError() after a launch -> JTMOE_OK or JTMOE_ELAUNCH (message set).
+int check_launch(const char* what);
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline size_t dtype_bytes(int dtype) { return dtype == JTMOE_F32 ? 4 : 2; }
+inline bool dtype_ok(int dtype) { return dtype == JTMOE_BF16 || dtype == JTMOE_F32; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- optional per-stage timing (only jtmoe_moe_forward_timed installs a timer) ----
+enum Stage {
+  kStageBegin = 0,
+  kStageRouter,
+  kStageDispatchMeta,
+  kStageDispatchRows,
+  kStageGateUp,
+  kStageDown,
+  kStageSharedGateUp,
+  kStageSharedDown,
+  kStageCombine,
+  kStageCount
+};
+struct StageTimer {
+  hipEvent_t ev[kStageCount];
+};
+extern thread_local StageTimer* g_stage_timer;
+// records the event that closes `stage` on `s`; a no-op unless a timer is installed
+inline void stage_mark(int stage, hipStream_t s) {
+  if (g_stage_timer) (void)hipEventRecord(g_stage_timer->ev[stage], s);
+}
+
+#define JT_REQUIRE(cond, ...)                          \
+  do {                                                 \
+    if (!(cond)) return ::jtmoe::fail(JTMOE_EINVAL, __VA_ARGS__); \
+  } while (0)
+
+// ---- device side: element types --------------------------------------------
+// bf16 values travel as raw 16-bit patterns; fp32 as float.
+struct bf16_raw {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bit pattern (NaN stays a quiet NaN)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<float> {
+  static constexpr bool is_bf16 = false;
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+template <>
+struct Elem<bf16_raw> {
+  static constexpr bool is_bf16 = true;
+  static __device__ __forceinline__ float load(const bf16_raw* p) { return bf16_bits_to_f32(p->bits); }
+  static __device__ __forceinline__ void store(bf16_raw* p, float v) { p->bits = (uint16_t)f32_to_bf16_bits(v); }
+  static __device__ __forceinline__ float round(float v) { return round_to_bf16(v); }
+};
+
+constexpr int kWave = 64;
+
+}  // namespace jtmoe

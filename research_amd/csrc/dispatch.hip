@@ -1,0 +1,236 @@
+// Token dispatch: per-expert histogram, exclusive prefix sum, the stable
+// permutation of assignments into expert-contiguous order with its inverse, and
+// the row gather into expert-major order.
+//
+// Follows local_dispatch of the reference at ep_size == 1 (moe.py:583-602):
+//   source_order = argsort(ids, stable)      inverse = argsort(source_order)
+//   group_sizes  = histogram(ids)            offsets = cumsum(group_sizes) - group_sizes
+//   packed_x[j]  = x[source_order[j] / K]
+//
+// The permutation is a counting sort whose positions come from an exclusive scan
+// over (expert-major, chunk-minor) partial histograms, so it is stable and
+// deterministic: no atomics decide a position.
+#include "common.hpp"
+
+namespace jtmoe {
+namespace {
+
+constexpr int kDispThreads = 256;
+constexpr int kDispWaves = kDispThreads / kWave;
+constexpr int kDispIters = 4;
+constexpr int kDispChunk = kDispThreads * kDispIters;  // assignments per workgroup
+
+inline int dispatch_chunks(int64_t A) { return (int)((A + kDispChunk - 1) / kDispChunk); }
+
+// pass 1: partial[e * nchunks + chunk] = #{a in chunk : ids[a] == e}
+__global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(const int32_t* __restrict__ ids, int A, int E,
+                                                                     int nchunks, int* __restrict__ partial) {
+  extern __shared__ int hist[];
+  for (int e = threadIdx.x; e < E; e += kDispThreads) hist[e] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kDispChunk;
+#pragma unroll
+  for (int it = 0; it < kDispIters; ++it) {
+    const int a = base + it * kDispThreads + threadIdx.x;
+    if (a < A) {
+      const int id = ids[a];
+      if (id >= 0 && id < E) atomicAdd(&hist[id], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kDispThreads) partial[(size_t)e * nchunks + blockIdx.x] = hist[e];
+}
+
+// pass 2 (one workgroup): in-place exclusive scan of partial[0 .. E*nchunks),
+// then group_sizes / offsets per expert.
+constexpr int kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void dispatch_scan_kernel(int* __restrict__ partial, int E, int nchunks,
+                                                                     int32_t* __restrict__ group_sizes,
+                                                                     int32_t* __restrict__ offsets) {
+  __shared__ int sums[kScanThreads];
+  __shared__ int total_s;
+  const int n = E * nchunks;
+  const int per = (n + kScanThreads - 1) / kScanThreads;
+  const int lo = min(n, (int)threadIdx.x * per), hi = min(n, lo + per);
+  int local = 0;
+  for (int i = lo; i < hi; ++i) local += partial[i];
+  sums[threadIdx.x] = local;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over the 1024 thread sums
+  for (int d = 1; d < kScanThreads; d <<= 1) {
+    const int v = (int)threadIdx.x >= d ? sums[threadIdx.x - d] : 0;
+    __syncthreads();
+    sums[threadIdx.x] += v;
+    __syncthreads();
+  }
+  int run = sums[threadIdx.x] - local;
+  if (threadIdx.x == kScanThreads - 1) total_s = sums[threadIdx.x];
+  for (int i = lo; i < hi; ++i) {
+    const int v = partial[i];
+    partial[i] = run;
+    run += v;
+  }
+  __syncthreads();
+  const int total = total_s;
+  for (int e = threadIdx.x; e < E; e += kScanThreads) {
+    const int start = partial[(size_t)e * nchunks];
+    const int next = (e + 1 < E) ? partial[(size_t)(e + 1) * nchunks] : total;
+    offsets[e] = start;
+    group_sizes[e] = next - start;
+  }
+}
+
+// pass 3: stable rank of every assignment inside its chunk + the chunk's base.
+__global__ __launch_bounds__(kDispThreads) void dispatch_rank_kernel(const int32_t* __restrict__ ids, int A, int E,
+                                                                     int nchunks, const int* __restrict__ base_g,
+                                                                     int32_t* __restrict__ source_order,
+                                                                     int32_t* __restrict__ inverse) {
+  extern __shared__ int smem[];
+  int* cursor = smem;         // [E] next free packed row of expert e for this chunk
+  int* wavehist = smem + E;   // [kDispWaves][E]
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  for (int e = tid; e < E; e += kDispThreads) cursor[e] = base_g[(size_t)e * nchunks + blockIdx.x];
+  for (int i = tid; i < kDispWaves * E; i += kDispThreads) wavehist[i] = 0;
+  __syncthreads();
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  const int base = blockIdx.x * kDispChunk;
+  for (int it = 0; it < kDispIters; ++it) {
+    const int a = base + it * kDispThreads + tid;
+    int id = -1;
+    if (a < A) {
+      id = ids[a];
+      if (id < 0 || id >= E) id = -1;
+    }
+    const bool valid = id >= 0;
+    // lanes of this wave holding the same expert id
+    unsigned long long peers = __ballot(valid);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (id >> b) & 1;
+      const unsigned long long m = __ballot(valid && bit);
+      peers &= bit ? m : ~m;
+    }
+    const unsigned long long lt = (1ull << lane) - 1ull;
+    const int rank = __popcll(peers & lt);
+    if (valid && rank == 0) wavehist[wave * E + id] = __popcll(peers);
+    __syncthreads();
+    if (valid) {
+      int pos = cursor[id] + rank;
+      for (int w = 0; w < wave; ++w) pos += wavehist[w * E + id];
+      inverse[a] = pos;
+      source_order[pos] = a;
+    } else if (a < A) {
+      inverse[a] = -1;
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += kDispThreads) {
+      int add = 0;
+#pragma unroll
+      for (int w = 0; w < kDispWaves; ++w) {
+        add += wavehist[w * E + e];
+        wavehist[w * E + e] = 0;
+      }
+      cursor[e] += add;
+    }
+    __syncthreads();
+  }
+}
+
+// pass 4: token-major row scatter; each token row is read once and written to
+// its K packed positions.  V is the vector type moved per lane.
+template <typename V>
+__global__ __launch_bounds__(256) void dispatch_rows_kernel(const V* __restrict__ x, const int32_t* __restrict__ inverse,
+                                                            int tokens, int K, int A, int row_vecs,
+                                                            V* __restrict__ packed_x) {
+  const int rows_per_block = blockDim.y;
+  const int t = blockIdx.x * rows_per_block + threadIdx.y;
+  if (t >= tokens) return;
+  const V* src = x + (size_t)t * row_vecs;
+  for (int v0 = threadIdx.x; v0 < row_vecs; v0 += blockDim.x * 4) {
+    V r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int v = v0 + j * blockDim.x;
+      if (v < row_vecs) r[j] = src[v];
+    }
+    for (int s = 0; s < K; ++s) {
+      const int pos = inverse[(size_t)t * K + s];
+      if (pos < 0 || pos >= A) continue;
+      V* dst = packed_x + (size_t)pos * row_vecs;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int v = v0 + j * blockDim.x;
+        if (v < row_vecs) dst[v] = r[j];
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace jtmoe
+
+using namespace jtmoe;
+
+extern "C" size_t jtmoe_dispatch_workspace_bytes(int64_t A, int64_t E) {
+  if (A < 0 || E <= 0) return 0;
+  const size_t chunks = (size_t)dispatch_chunks(A > 0 ? A : 1);
+  return align_up(chunks * (size_t)E * sizeof(int), 256);
+}
+
+extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E, int64_t K,
+                              int dtype, int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
+                              int32_t* inverse, void* packed_x, void* workspace, size_t workspace_bytes,
+                              void* stream) {
+  clear_error();
+  JT_REQUIRE(dtype_ok(dtype), "dispatch: unknown dtype %d", dtype);
+  JT_REQUIRE(T >= 0 && K > 0 && E > 0, "dispatch: T=%lld K=%lld E=%lld out of range", (long long)T, (long long)K,
+             (long long)E);
+  if (E > JTMOE_MAX_EXPERTS) return fail(JTMOE_EUNSUPPORTED, "dispatch: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  const int64_t A = T * K;
+  JT_REQUIRE(A < ((int64_t)1 << 31), "dispatch: T*K exceeds int32");
+  JT_REQUIRE(group_sizes && offsets && workspace, "dispatch: null pointer argument");
+  JT_REQUIRE(A == 0 || (expert_ids && source_order && inverse), "dispatch: null pointer argument");
+  JT_REQUIRE(x == nullptr || (H > 0 && packed_x != nullptr), "dispatch: x given without H or packed_x");
+  JT_REQUIRE(x == nullptr || H * (int64_t)dtype_bytes(dtype) < ((int64_t)1 << 31), "dispatch: row too long");
+  if (workspace_bytes < jtmoe_dispatch_workspace_bytes(A, E))
+    return fail(JTMOE_EWORKSPACE, "dispatch: workspace %zu < %zu bytes", workspace_bytes,
+                jtmoe_dispatch_workspace_bytes(A, E));
+  hipStream_t s = as_stream(stream);
+  const int nchunks = dispatch_chunks(A > 0 ? A : 1);
+  int* partial = static_cast<int*>(workspace);
+  dispatch_hist_kernel<<<nchunks, kDispThreads, (size_t)E * sizeof(int), s>>>(expert_ids, (int)A, (int)E, nchunks,
+                                                                              partial);
+  dispatch_scan_kernel<<<1, kScanThreads, 0, s>>>(partial, (int)E, nchunks, group_sizes, offsets);
+  if (A > 0) {
+    dispatch_rank_kernel<<<nchunks, kDispThreads, (size_t)E * (1 + kDispWaves) * sizeof(int), s>>>(
+        expert_ids, (int)A, (int)E, nchunks, partial, source_order, inverse);
+    stage_mark(kStageDispatchMeta, s);
+    if (x != nullptr) {
+      const size_t row_bytes = (size_t)H * dtype_bytes(dtype);
+      const bool vec16 = row_bytes % 16 == 0 && aligned16(x) && aligned16(packed_x);
+      if (vec16) {
+        const int row_vecs = (int)(row_bytes / 16);
+        // one wave per row for short rows, up to 256 lanes for long ones
+        int bx = 64;
+        while (bx < 256 && bx * 4 < row_vecs) bx *= 2;
+        dim3 block(bx, 256 / bx);
+        const int grid = (int)((T + block.y - 1) / block.y);
+        dispatch_rows_kernel<uint4><<<grid, block, 0, s>>>(static_cast<const uint4*>(x), inverse, (int)T, (int)K,
+                                                           (int)A, row_vecs, static_cast<uint4*>(packed_x));
+      } else if (dtype == JTMOE_BF16) {
+        dim3 block(64, 4);
+        const int grid = (int)((T + block.y - 1) / block.y);
+        dispatch_rows_kernel<uint16_t><<<grid, block, 0, s>>>(static_cast<const uint16_t*>(x), inverse, (int)T, (int)K,
+                                                              (int)A, (int)H, static_cast<uint16_t*>(packed_x));
+      } else {
+        dim3 block(64, 4);
+        const int grid = (int)((T + block.y - 1) / block.y);
+        dispatch_rows_kernel<uint32_t><<<grid, block, 0, s>>>(static_cast<const uint32_t*>(x), inverse, (int)T, (int)K,
+                                                              (int)A, (int)H, static_cast<uint32_t*>(packed_x));
+      }
+    }
+  }
+  if (A == 0) stage_mark(kStageDispatchMeta, s);
+  stage_mark(kStageDispatchRows, s);
+  return check_launch("dispatch");
+}

@@ -1,0 +1,241 @@
+// Grouped SwiGLU expert FFN: two grouped GEMM launches over variable-size,
+// expert-contiguous row groups.
+//
+// Follows the three jax.lax.ragged_dot calls of the reference and the SwiGLU
+// between them (moe.py:638-641), and SharedSwiGLU.__call__ (moe.py:361-364) as
+// the one-group dense case:
+//   launch 1 (dual):  act = round(silu(round(X Wg[e])) * round(X Wu[e]))   [rows, I]
+//   launch 2:         Y   = round(act Wd[e])                                [rows, H]
+// `round` is the rounding to the compute dtype (identity for fp32); products
+// are accumulated in fp32 on the matrix cores (v_mfma_f32_32x32x16_bf16 for
+// bf16, v_mfma_f32_32x32x2_f32 for fp32).
+#include "common.hpp"
+
+namespace jtmoe {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+// Row range of one m-tile.  Groups are the experts' contiguous row ranges; tile
+// `mt` counts m-tiles expert by expert (ceil(group_size / BM) each).
+struct TileRows {
+  int expert;
+  int row0;  // first packed row of the tile
+  int rows;  // valid rows in the tile (0 = no such tile)
+};
+
+__device__ __forceinline__ TileRows find_tile(int mt, int BM, const int32_t* __restrict__ group_sizes,
+                                              const int32_t* __restrict__ offsets, int E, int dense_rows) {
+  TileRows r;
+  r.expert = 0;
+  r.row0 = 0;
+  r.rows = 0;
+  if (group_sizes == nullptr) {
+    const int row0 = mt * BM;
+    if (row0 < dense_rows) {
+      r.row0 = row0;
+      r.rows = min(BM, dense_rows - row0);
+    }
+    return r;
+  }
+  int first = 0;
+  for (int e = 0; e < E; ++e) {
+    const int n = group_sizes[e];
+    const int tiles = (n + BM - 1) / BM;
+    if (mt < first + tiles) {
+      const int local = mt - first;
+      r.expert = e;
+      r.row0 = offsets[e] + local * BM;
+      r.rows = min(BM, n - local * BM);
+      return r;
+    }
+    first += tiles;
+  }
+  return r;
+}
+
+__device__ __forceinline__ float silu_fast(float g) { return g / (1.0f + __expf(-g)); }
+
+// ---------------------------------------------------------------------------
+// Generic kernel: any shape, any alignment, both dtypes.  64x64x32 tiles, four
+// waves (2x2), each owning one 32x32 accumulator tile (two when kDual).
+// Operands are staged element by element through LDS with bounds checks; B is
+// transposed on the way in so that both MFMA operands are k-contiguous.
+// ---------------------------------------------------------------------------
+constexpr int GBM = 64, GBN = 64, GBK = 32;
+constexpr int GPAD = 8;  // elements; keeps 16-byte alignment of bf16 rows
+
+template <typename T>
+__device__ __forceinline__ void mfma_tile(const T* __restrict__ a_row, const T* __restrict__ b_row, int khalf,
+                                          f32x16_t& acc);
+
+// a_row / b_row point at the k = 0 element of this lane's A row / B column in LDS
+template <>
+__device__ __forceinline__ void mfma_tile<bf16_raw>(const bf16_raw* __restrict__ a_row,
+                                                    const bf16_raw* __restrict__ b_row, int khalf, f32x16_t& acc) {
+#pragma unroll
+  for (int kk = 0; kk < GBK / 16; ++kk) {
+    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(a_row + kk * 16 + khalf * 8);
+    const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(b_row + kk * 16 + khalf * 8);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+  }
+}
+
+template <>
+__device__ __forceinline__ void mfma_tile<float>(const float* __restrict__ a_row, const float* __restrict__ b_row,
+                                                 int khalf, f32x16_t& acc) {
+#pragma unroll
+  for (int kk = 0; kk < GBK / 2; ++kk) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_row[kk * 2 + khalf], b_row[kk * 2 + khalf], acc, 0, 0, 0);
+  }
+}
+
+template <typename T, bool kDual>
+__global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(
+    const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
+    const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E, int dense_rows, int Kdim,
+    int N, int ntiles_n) {
+  __shared__ __align__(16) T As[GBM][GBK + GPAD];
+  __shared__ __align__(16) T Bs0[GBN][GBK + GPAD];
+  __shared__ __align__(16) T Bs1[kDual ? GBN : 1][GBK + GPAD];
+
+  const int mt = blockIdx.x / ntiles_n;
+  const int nt = blockIdx.x - mt * ntiles_n;
+  const TileRows tr = find_tile(mt, GBM, group_sizes, offsets, E, dense_rows);
+  if (tr.rows <= 0) return;
+  const int n0 = nt * GBN;
+  const size_t wofs = (size_t)tr.expert * Kdim * N;
+  const T* Bg0 = B0 + wofs;
+  const T* Bg1 = kDual ? B1 + wofs : nullptr;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int frag_row = lane & 31, khalf = lane >> 5;
+
+  f32x16_t acc0, acc1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    acc0[i] = 0.0f;
+    acc1[i] = 0.0f;
+  }
+
+  T zero;
+  __builtin_memset(&zero, 0, sizeof(T));
+
+  for (int k0 = 0; k0 < Kdim; k0 += GBK) {
+    for (int idx = tid; idx < GBM * GBK; idx += 256) {
+      const int r = idx / GBK, c = idx - r * GBK;
+      const int gk = k0 + c;
+      T v = zero;
+      if (r < tr.rows && gk < Kdim) v = A[(size_t)(tr.row0 + r) * Kdim + gk];
+      As[r][c] = v;
+    }
+    for (int idx = tid; idx < GBK * GBN; idx += 256) {
+      const int k = idx / GBN, n = idx - k * GBN;
+      const int gk = k0 + k, gn = n0 + n;
+      const bool ok = gk < Kdim && gn < N;
+      Bs0[n][k] = ok ? Bg0[(size_t)gk * N + gn] : zero;
+      if (kDual) Bs1[n][k] = ok ? Bg1[(size_t)gk * N + gn] : zero;
+    }
+    __syncthreads();
+    const T* a_row = &As[wm * 32 + frag_row][0];
+    mfma_tile<T>(a_row, &Bs0[wn * 32 + frag_row][0], khalf, acc0);
+    if (kDual) mfma_tile<T>(a_row, &Bs1[wn * 32 + frag_row][0], khalf, acc1);
+    __syncthreads();
+  }
+
+  // 32x32 accumulator layout: value i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32
+  const int col = n0 + wn * 32 + (lane & 31);
+  if (col < N) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = wm * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+      if (r < tr.rows) {
+        float v;
+        if (kDual) {
+          const float g = Elem<T>::round(acc0[i]);
+          const float u = Elem<T>::round(acc1[i]);
+          v = silu_fast(g) * u;
+        } else {
+          v = acc0[i];
+        }
+        Elem<T>::store(C + (size_t)(tr.row0 + r) * N + col, v);
+      }
+    }
+  }
+}
+
+// upper bound on the number of m-tiles when the group sizes live on the device
+inline int64_t max_m_tiles(int64_t rows, int64_t groups, int BM) {
+  return (rows + BM - 1) / BM + (groups < rows ? groups : rows);
+}
+
+template <typename T>
+int launch_pair(const void* x, const void* gate, const void* up, const void* down, const int32_t* group_sizes,
+                const int32_t* offsets, int64_t rows, int64_t H, int64_t I, int64_t E, void* act, void* y,
+                hipStream_t stream, int first_stage) {
+  const bool dense = group_sizes == nullptr;
+  const int64_t mtiles = dense ? (rows + GBM - 1) / GBM : max_m_tiles(rows, E, GBM);
+  if (mtiles == 0) return JTMOE_OK;
+  {
+    const int64_t nt = (I + GBN - 1) / GBN;
+    if (mtiles * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
+    grouped_gemm_generic_kernel<T, true><<<(unsigned)(mtiles * nt), 256, 0, stream>>>(
+        static_cast<const T*>(x), static_cast<const T*>(gate), static_cast<const T*>(up), static_cast<T*>(act),
+        group_sizes, offsets, (int)E, (int)rows, (int)H, (int)I, (int)nt);
+  }
+  stage_mark(first_stage, stream);
+  {
+    const int64_t nt = (H + GBN - 1) / GBN;
+    if (mtiles * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
+    grouped_gemm_generic_kernel<T, false><<<(unsigned)(mtiles * nt), 256, 0, stream>>>(
+        static_cast<const T*>(act), static_cast<const T*>(down), nullptr, static_cast<T*>(y), group_sizes, offsets,
+        (int)E, (int)rows, (int)I, (int)H, (int)nt);
+  }
+  stage_mark(first_stage + 1, stream);
+  return check_launch("grouped gemm");
+}
+
+int validate_gemm(const char* what, int64_t rows, int64_t H, int64_t I, int64_t E, int dtype) {
+  JT_REQUIRE(dtype_ok(dtype), "%s: unknown dtype %d", what, dtype);
+  JT_REQUIRE(rows >= 0 && rows < ((int64_t)1 << 31), "%s: row count %lld out of range", what, (long long)rows);
+  JT_REQUIRE(H > 0 && I > 0 && E > 0, "%s: H=%lld I=%lld E=%lld out of range", what, (long long)H, (long long)I,
+             (long long)E);
+  JT_REQUIRE(H < ((int64_t)1 << 24) && I < ((int64_t)1 << 24), "%s: H or I too large", what);
+  return JTMOE_OK;
+}
+
+}  // namespace
+}  // namespace jtmoe
+
+using namespace jtmoe;
+
+extern "C" int jtmoe_grouped_swiglu(const void* packed_x, const void* gate, const void* up, const void* down,
+                                    const int32_t* group_sizes, const int32_t* offsets, int64_t A, int64_t H,
+                                    int64_t I, int64_t E, int dtype, void* act, void* packed_y, void* stream) {
+  clear_error();
+  int rc = validate_gemm("grouped_swiglu", A, H, I, E, dtype);
+  if (rc) return rc;
+  if (E > JTMOE_MAX_EXPERTS) return fail(JTMOE_EUNSUPPORTED, "grouped_swiglu: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  if (A == 0) return JTMOE_OK;
+  JT_REQUIRE(packed_x && gate && up && down && group_sizes && offsets && act && packed_y,
+             "grouped_swiglu: null pointer argument");
+  hipStream_t s = as_stream(stream);
+  if (dtype == JTMOE_BF16)
+    return launch_pair<bf16_raw>(packed_x, gate, up, down, group_sizes, offsets, A, H, I, E, act, packed_y, s, kStageGateUp);
+  return launch_pair<float>(packed_x, gate, up, down, group_sizes, offsets, A, H, I, E, act, packed_y, s, kStageGateUp);
+}
+
+extern "C" int jtmoe_shared_swiglu(const void* x, const void* gate, const void* up, const void* down, int64_t T,
+                                   int64_t H, int64_t Is, int dtype, void* act, void* shared_y, void* stream) {
+  clear_error();
+  int rc = validate_gemm("shared_swiglu", T, H, Is, 1, dtype);
+  if (rc) return rc;
+  if (T == 0) return JTMOE_OK;
+  JT_REQUIRE(x && gate && up && down && act && shared_y, "shared_swiglu: null pointer argument");
+  hipStream_t s = as_stream(stream);
+  if (dtype == JTMOE_BF16)
+    return launch_pair<bf16_raw>(x, gate, up, down, nullptr, nullptr, T, H, Is, 1, act, shared_y, s, kStageSharedGateUp);
+  return launch_pair<float>(x, gate, up, down, nullptr, nullptr, T, H, Is, 1, act, shared_y, s, kStageSharedGateUp);
+}

@@ -1,0 +1,331 @@
+// Router: logits -> sigmoid -> (+bias) top-k -> renormalised weights, plus the
+// per-expert counts / importance of the router statistics.
+//
+// Follows SigmoidTopKRouter.__call__ (reference moe.py:131-147) and the two
+// vector outputs of _router_stats (moe.py:802-805).
+//
+// This file is compiled with floating-point contraction OFF and correctly
+// rounded fp32 division: everything after the logits is a fixed sequence of
+// IEEE-754 single operations, so the routing decision is a pure function of the
+// logits and can be reproduced bit for bit on a CPU.
+#include "common.hpp"
+
+#include <mutex>
+
+namespace jtmoe {
+namespace {
+
+constexpr int kRouterTokens = 64;    // tokens per workgroup
+constexpr int kRouterThreads = 256;  // 4 lanes per token in the selection phase
+constexpr float kFixedScale = 4294967296.0f;  // importance is summed in 32.32 fixed point
+
+// ---- fully specified fp32 sigmoid ------------------------------------------
+__device__ __forceinline__ float exp_fixed(float x) {
+#pragma clang fp contract(off)
+  const float n = rintf(x * 1.4426950408889634f);
+  float r = x - n * 0.693145751953125f;
+  r = r - n * 1.428606765330187e-06f;
+  float p = 1.9875691500e-4f;
+  p = p * r;
+  p = p + 1.3981999507e-3f;
+  p = p * r;
+  p = p + 8.3334519073e-3f;
+  p = p * r;
+  p = p + 4.1665795894e-2f;
+  p = p * r;
+  p = p + 1.6666665459e-1f;
+  p = p * r;
+  p = p + 5.0000001201e-1f;
+  const float rr = r * r;
+  p = p * rr;
+  p = p + r;
+  p = p + 1.0f;
+  return ldexpf(p, (int)n);
+}
+
+__device__ __forceinline__ float sigmoid_fixed(float z) {
+#pragma clang fp contract(off)
+  float t = -z;
+  t = fmaxf(t, -86.0f);
+  t = fminf(t, 86.0f);
+  const float e = exp_fixed(t);
+  return 1.0f / (1.0f + e);
+}
+
+// ---- scratch ----------------------------------------------------------------
+struct RouterScratch {
+  unsigned long long* imp;  // [E] 32.32 fixed point
+  int* cnt;                 // [E]
+};
+
+__host__ __device__ inline RouterScratch router_scratch(void* ws, int E) {
+  RouterScratch s;
+  s.imp = reinterpret_cast<unsigned long long*>(ws);
+  s.cnt = reinterpret_cast<int*>(s.imp + E);
+  return s;
+}
+
+__global__ void router_zero_kernel(void* ws, int E) {
+  RouterScratch s = router_scratch(ws, E);
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    s.imp[e] = 0ull;
+    s.cnt[e] = 0;
+  }
+}
+
+__global__ void router_finalize_kernel(const void* ws, int E, float* counts, float* importance) {
+  RouterScratch s = router_scratch(const_cast<void*>(ws), E);
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    counts[e] = (float)s.cnt[e];
+    importance[e] = (float)((double)s.imp[e] * (1.0 / 4294967296.0));
+  }
+}
+
+// ---- LDS layout of one workgroup ----------------------------------------------
+struct RouterSmem {
+  float* tile;       // [kRouterTokens][E+1] logits, then scores
+  float* bias;       // [E]
+  float* top_score;  // [kRouterTokens][K]
+  int* top_id;       // [kRouterTokens][K]
+  int* cnt;          // [E]
+  unsigned long long* imp;  // [E]
+};
+
+__host__ __device__ inline size_t router_smem_bytes(int E, int K) {
+  size_t n = 0;
+  n += (size_t)E * 8;                        // imp (first: 8-byte aligned)
+  n += (size_t)kRouterTokens * (E + 1) * 4;  // tile
+  n += (size_t)E * 4;                        // bias
+  n += (size_t)kRouterTokens * K * 4 * 2;    // top_score, top_id
+  n += (size_t)E * 4;                        // cnt
+  return n;
+}
+
+__device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, int K) {
+  RouterSmem s;
+  s.imp = reinterpret_cast<unsigned long long*>(base);
+  s.tile = reinterpret_cast<float*>(s.imp + E);
+  s.bias = s.tile + kRouterTokens * (E + 1);
+  s.top_score = s.bias + E;
+  s.top_id = reinterpret_cast<int*>(s.top_score + kRouterTokens * K);
+  s.cnt = s.top_id + kRouterTokens * K;
+  return s;
+}
+
+// Everything after the logits tile is in LDS.  `T` is the output element type of
+// the weights.
+template <typename T>
+__device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ bias_g, int t0, int tokens,
+                                int E, int K, float route_scale, int32_t* __restrict__ ids_out,
+                                T* __restrict__ weights_out, float* __restrict__ scores_out,
+                                float* __restrict__ logits_out, RouterScratch g) {
+#pragma clang fp contract(off)
+  const int tid = threadIdx.x;
+  const int stride = E + 1;
+  const int nrows = min(kRouterTokens, tokens - t0);
+
+  for (int e = tid; e < E; e += kRouterThreads) {
+    sm.bias[e] = bias_g ? bias_g[e] : 0.0f;
+    sm.cnt[e] = 0;
+    sm.imp[e] = 0ull;
+  }
+  // logits -> scores (in place), both written out row-major
+  for (int idx = tid; idx < nrows * E; idx += kRouterThreads) {
+    const int t = idx / E, e = idx - t * E;
+    const float z = sm.tile[t * stride + e];
+    if (logits_out) logits_out[(size_t)(t0 + t) * E + e] = z;
+    const float s = sigmoid_fixed(z);
+    sm.tile[t * stride + e] = s;
+    scores_out[(size_t)(t0 + t) * E + e] = s;
+  }
+  __syncthreads();
+
+  // selection: 4 lanes per token, each owning a contiguous quarter of the experts
+  const int t = tid >> 2, q = tid & 3;
+  const int eq = (E + 3) >> 2;
+  const int e_begin = q * eq;
+  const bool row_ok = t < nrows;
+  unsigned long long taken = 0ull;
+  const float* row = sm.tile + t * stride;
+  for (int r = 0; r < K; ++r) {
+    float best_v = 0.0f;
+    int best_e = -1;
+    if (row_ok) {
+      for (int j = 0; j < eq; ++j) {
+        const int e = e_begin + j;
+        if (e < E && !((taken >> j) & 1ull)) {
+          const float v = row[e] + sm.bias[e];
+          if (best_e < 0 || v > best_v) {
+            best_v = v;
+            best_e = e;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 1; m <= 2; m <<= 1) {
+      const float ov = __shfl_xor(best_v, m, 4);
+      const int oe = __shfl_xor(best_e, m, 4);
+      const bool take = oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e));
+      if (take) {
+        best_v = ov;
+        best_e = oe;
+      }
+    }
+    if (row_ok) {
+      const int j = best_e - e_begin;
+      if (j >= 0 && j < eq) taken |= 1ull << j;
+      if (q == 0) {
+        sm.top_id[t * K + r] = best_e;
+        sm.top_score[t * K + r] = row[best_e];
+      }
+    }
+  }
+  // renormalise (lane 0 of the token; it wrote top_* itself)
+  if (row_ok && q == 0) {
+    float denom = sm.top_score[t * K];
+    for (int r = 1; r < K; ++r) denom = denom + sm.top_score[t * K + r];
+    denom = denom + 1e-20f;
+    for (int r = 0; r < K; ++r) {
+      const int e = sm.top_id[t * K + r];
+      float w = sm.top_score[t * K + r] / denom;
+      w = w * route_scale;
+      w = Elem<T>::round(w);
+      const size_t o = (size_t)(t0 + t) * K + r;
+      ids_out[o] = e;
+      Elem<T>::store(weights_out + o, w);
+      atomicAdd(&sm.cnt[e], 1);
+      atomicAdd(&sm.imp[e], (unsigned long long)(w * kFixedScale));
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += kRouterThreads) {
+    const int c = sm.cnt[e];
+    if (c) {
+      atomicAdd(&g.cnt[e], c);
+      atomicAdd(&g.imp[e], sm.imp[e]);
+    }
+  }
+}
+
+// Generic projection: any H, E; fp32 accumulation in k order.
+template <typename T, bool kFromLogits>
+__global__ __launch_bounds__(kRouterThreads) void router_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ logits_in,
+    const float* __restrict__ bias, int tokens, int H, int E, int K, float route_scale,
+    int32_t* __restrict__ ids, T* __restrict__ weights, float* __restrict__ scores,
+    float* __restrict__ logits_out, void* ws) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  RouterSmem sm = router_smem(smem_raw, E, K);
+  const int t0 = blockIdx.x * kRouterTokens;
+  const int nrows = min(kRouterTokens, tokens - t0);
+  const int stride = E + 1;
+  for (int idx = threadIdx.x; idx < nrows * E; idx += kRouterThreads) {
+    const int t = idx / E, e = idx - t * E;
+    float z;
+    if (kFromLogits) {
+      z = logits_in[(size_t)(t0 + t) * E + e];
+    } else {
+      const T* xr = x + (size_t)(t0 + t) * H;
+      float acc = 0.0f;
+      for (int k = 0; k < H; ++k) acc = fmaf(Elem<T>::load(xr + k), Elem<T>::load(w + (size_t)k * E + e), acc);
+      z = Elem<T>::round(acc);
+    }
+    sm.tile[t * stride + e] = z;
+  }
+  __syncthreads();
+  router_epilogue<T>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
+                     router_scratch(ws, E));
+}
+
+template <typename KernelT>
+int set_max_smem(KernelT kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return JTMOE_OK;
+  hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (err != hipSuccess) return fail(JTMOE_ELAUNCH, "hipFuncSetAttribute(router): %s", hipGetErrorString(err));
+  return JTMOE_OK;
+}
+
+template <typename T, bool kFromLogits>
+int launch_router(const void* x, const void* w, const float* logits_in, const float* bias, int64_t tokens,
+                  int64_t H, int64_t E, int64_t K, double route_scale, int32_t* ids, void* weights,
+                  float* scores, float* counts, float* importance, float* logits_out, void* ws,
+                  hipStream_t stream) {
+  const size_t smem = router_smem_bytes((int)E, (int)K);
+  if (smem > 160 * 1024) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
+  auto kernel = router_kernel<T, kFromLogits>;
+  int rc = set_max_smem(kernel, smem);
+  if (rc) return rc;
+  router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
+  if (tokens > 0) {
+    const int blocks = (int)((tokens + kRouterTokens - 1) / kRouterTokens);
+    kernel<<<blocks, kRouterThreads, smem, stream>>>(
+        static_cast<const T*>(x), static_cast<const T*>(w), logits_in, bias, (int)tokens, (int)H, (int)E, (int)K,
+        (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws);
+  }
+  router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
+  return check_launch("router");
+}
+
+int validate_router(int64_t T, int64_t H, int64_t E, int64_t K, double route_scale, int dtype, bool need_h) {
+  JT_REQUIRE(dtype_ok(dtype), "router: unknown dtype %d", dtype);
+  JT_REQUIRE(T >= 0 && T <= (int64_t)1 << 30, "router: token count %lld out of range", (long long)T);
+  JT_REQUIRE(!need_h || (H > 0 && H <= (int64_t)1 << 20), "router: hidden size %lld out of range", (long long)H);
+  JT_REQUIRE(E > 0 && K > 0 && K <= E, "router top_k must be positive and <= num_experts (E=%lld K=%lld)",
+             (long long)E, (long long)K);
+  JT_REQUIRE(route_scale > 0.0, "router route_scale must be positive, got %g", route_scale);
+  if (E > JTMOE_MAX_EXPERTS) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  if (K > JTMOE_MAX_TOP_K) return fail(JTMOE_EUNSUPPORTED, "router: K=%lld exceeds %d", (long long)K, JTMOE_MAX_TOP_K);
+  JT_REQUIRE(T * E < ((int64_t)1 << 31) && T * K < ((int64_t)1 << 31), "router: T*E or T*K exceeds int32");
+  return JTMOE_OK;
+}
+
+}  // namespace
+}  // namespace jtmoe
+
+using namespace jtmoe;
+
+extern "C" size_t jtmoe_router_workspace_bytes(int64_t E) {
+  if (E <= 0) return 0;
+  return align_up((size_t)E * 12, 256);
+}
+
+extern "C" int jtmoe_router(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H,
+                            int64_t E, int64_t K, double route_scale, int dtype, int32_t* expert_ids,
+                            void* weights, float* scores, float* expert_counts, float* importance, float* logits,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  int rc = validate_router(T, H, E, K, route_scale, dtype, true);
+  if (rc) return rc;
+  JT_REQUIRE(w_router && expert_counts && importance && workspace, "router: null pointer argument");
+  JT_REQUIRE(T == 0 || (x && expert_ids && weights && scores), "router: null pointer argument");
+  if (workspace_bytes < jtmoe_router_workspace_bytes(E))
+    return fail(JTMOE_EWORKSPACE, "router: workspace %zu < %zu bytes", workspace_bytes, jtmoe_router_workspace_bytes(E));
+  hipStream_t s = as_stream(stream);
+  if (dtype == JTMOE_BF16)
+    return launch_router<bf16_raw, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids,
+                                          weights, scores, expert_counts, importance, logits, workspace, s);
+  return launch_router<float, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
+                                     scores, expert_counts, importance, logits, workspace, s);
+}
+
+extern "C" int jtmoe_router_from_logits(const float* logits, const float* expert_bias, int64_t T, int64_t E,
+                                        int64_t K, double route_scale, int dtype, int32_t* expert_ids,
+                                        void* weights, float* scores, float* expert_counts, float* importance,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  int rc = validate_router(T, 1, E, K, route_scale, dtype, false);
+  if (rc) return rc;
+  JT_REQUIRE(expert_counts && importance && workspace, "router_from_logits: null pointer argument");
+  JT_REQUIRE(T == 0 || (logits && expert_ids && weights && scores), "router_from_logits: null pointer argument");
+  if (workspace_bytes < jtmoe_router_workspace_bytes(E))
+    return fail(JTMOE_EWORKSPACE, "router_from_logits: workspace %zu < %zu bytes", workspace_bytes,
+                jtmoe_router_workspace_bytes(E));
+  hipStream_t s = as_stream(stream);
+  if (dtype == JTMOE_BF16)
+    return launch_router<bf16_raw, true>(nullptr, nullptr, logits, expert_bias, T, 0, E, K, route_scale, expert_ids,
+                                         weights, scores, expert_counts, importance, nullptr, workspace, s);
+  return launch_router<float, true>(nullptr, nullptr, logits, expert_bias, T, 0, E, K, route_scale, expert_ids, weights,
+                                    scores, expert_counts, importance, nullptr, workspace, s);
+}

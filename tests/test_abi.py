@@ -1,0 +1,101 @@
+"""CPU-side checks of the drop-in boundary: the library loads, exports every
+symbol the header declares, its pure host functions answer, and the loader /
+wrappers fail loudly (no fallback) on a bad artefact or bad arguments."""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+import re
+import shutil
+
+import pytest
+
+from research_amd import _ffi, build
+from research_amd.errors import ContractError
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def header_symbols() -> set[str]:
+    text = (ROOT / "include" / "jtmoe.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(jtmoe_[a-z0-9_]+)\s*\(", text))
+
+
+def test_header_and_binding_agree():
+    assert header_symbols() == set(_ffi.PROTOTYPES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _ffi.load_library()
+    for name in header_symbols():
+        assert hasattr(lib, name), name
+    assert lib.jtmoe_version() == 1
+    assert _ffi.last_error(lib) == ""
+
+
+def test_workspace_sizing_is_pure_host_arithmetic():
+    lib = _ffi.load_library()
+    T, H, E, K, I, Is = 16384, 2048, 64, 8, 1408, 2816
+    total = lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, _ffi.JTMOE_BF16)
+    A = T * K
+    payload = 2 * (A * H + A * I + A * H + T * Is + T * H)
+    assert payload <= total <= payload + 2**20
+    assert total % 256 == 0
+    assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, _ffi.JTMOE_F32) >= 2 * payload
+    assert lib.jtmoe_workspace_bytes(0, H, E, K, I, 0, _ffi.JTMOE_BF16) > 0
+    assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, 7) == 0  # unknown dtype
+    assert lib.jtmoe_router_workspace_bytes(E) >= 12 * E
+    assert lib.jtmoe_dispatch_workspace_bytes(A, E) >= 4 * E * ((A + 1023) // 1024)
+    assert lib.jtmoe_balance_workspace_bytes(8, E) >= 32
+
+
+def test_argument_errors_return_status_and_message_without_a_gpu():
+    lib = _ffi.load_library()
+    # validation happens before any launch: null pointers / bad attributes are reported, nothing runs
+    rc = lib.jtmoe_combine(None, None, None, None, 4, 8, 2, 9, None, None)
+    assert rc == -1 and "dtype" in _ffi.last_error(lib)
+    rc = lib.jtmoe_router(None, None, None, 4, 8, 4, 5, 1.0, _ffi.JTMOE_BF16, None, None, None, None, None, None,
+                          None, 0, None)
+    assert rc == -1 and "top_k" in _ffi.last_error(lib)
+    rc = lib.jtmoe_router(None, None, None, 4, 8, 4, 2, 0.0, _ffi.JTMOE_BF16, None, None, None, None, None, None,
+                          None, 0, None)
+    assert rc == -1 and "route_scale" in _ffi.last_error(lib)
+    rc = lib.jtmoe_router(None, None, None, 4, 8, 1024, 2, 1.0, _ffi.JTMOE_BF16, None, None, None, None, None, None,
+                          None, 0, None)
+    assert rc == -2
+    rc = lib.jtmoe_grouped_swiglu(None, None, None, None, None, None, 16, 8, 8, 2, _ffi.JTMOE_BF16, None, None, None)
+    assert rc == -1 and "null" in _ffi.last_error(lib)
+    rc = lib.jtmoe_moe_forward(*([None] * 9), 4, 8, 2, 1, 8, 0, 1.0, _ffi.JTMOE_BF16, *([None] * 10), None, 0, None)
+    assert rc == -1 and "workspace" in _ffi.last_error(lib)
+
+
+def test_loader_refuses_missing_or_stale_artifacts(tmp_path):
+    with pytest.raises(ContractError, match="manifest is missing"):
+        _ffi.shared_object_path(tmp_path)
+    src = build.cache_dir()
+    shutil.copy(src / build.LIBRARY_NAME, tmp_path / build.LIBRARY_NAME)
+    shutil.copy(src / build.MANIFEST_NAME, tmp_path / build.MANIFEST_NAME)
+    assert _ffi.shared_object_path(tmp_path).name == build.LIBRARY_NAME
+    with (tmp_path / build.LIBRARY_NAME).open("ab") as handle:
+        handle.write(b"\0")
+    with pytest.raises(ContractError, match="checksum mismatch"):
+        _ffi.shared_object_path(tmp_path)
+    (tmp_path / build.LIBRARY_NAME).unlink()
+    with pytest.raises(ContractError, match="is missing"):
+        _ffi.shared_object_path(tmp_path)
+    (tmp_path / build.MANIFEST_NAME).write_text("{not json")
+    with pytest.raises(ContractError, match="failed to parse"):
+        _ffi.shared_object_path(tmp_path)
+    (tmp_path / build.MANIFEST_NAME).write_text(json.dumps({"artifacts": {}}))
+    with pytest.raises(ContractError, match="does not contain"):
+        _ffi.shared_object_path(tmp_path)
+
+
+def test_manifest_records_the_build():
+    manifest = build.load_cache_manifest()
+    art = manifest["artifacts"]["moe"]["ffi"]
+    assert art["arch"] == "gfx950" and art["kind"] == "ffi"
+    assert set(art["sources"]) == set(build.SOURCE_FILES)
+    assert len(art["sha256"]) == 64 and art["bytes"] > 0

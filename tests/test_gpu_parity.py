@@ -1,0 +1,410 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle, on the GPU.
+
+Bars: expert ids, per-expert counts, offsets and the permutation are bit-exact;
+the routing decision is bit-exact given the same logits; combine is bit-exact
+given the same expert outputs; floating-point outputs of the matrix products
+are within max|y-ref|/max|ref| <= 2e-2 for bf16 (mean abs error printed) and
+1e-5-class for fp32.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from research_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+BF16_MAX_REL = 2e-2  # max|y-ref| / max|ref|
+F32_TOL = dict(rtol=2e-5, atol=2e-5)
+
+
+def dev(a: np.ndarray, gpu, dtype: str | None = None) -> torch.Tensor:
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    if dtype == "bf16":
+        t = t.to(torch.bfloat16)
+    return t.contiguous()
+
+
+def host(t: torch.Tensor) -> np.ndarray:
+    return t.detach().float().cpu().numpy() if t.dtype == torch.bfloat16 else t.detach().cpu().numpy()
+
+
+def rel_err(got: np.ndarray, ref: np.ndarray) -> float:
+    scale = float(np.max(np.abs(ref))) or 1.0
+    return float(np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)))) / scale
+
+
+def report(tag: str, got: np.ndarray, ref: np.ndarray) -> float:
+    r = rel_err(got, ref)
+    print(f"[parity] {tag}: max_rel={r:.3e} mean_abs={float(np.mean(np.abs(got - ref))):.3e}", flush=True)
+    return r
+
+
+# --------------------------------------------------------------------------
+# router
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize(
+    "tokens,experts,top_k,dtype,scale,use_bias",
+    [
+        (1, 3, 2, "f32", 1.0, False),
+        (65, 8, 2, "f32", 1.5, True),
+        (300, 16, 2, "bf16", 1.0, False),
+        (1000, 64, 8, "bf16", 2.5, True),
+        (513, 128, 8, "bf16", 1.0, True),
+        (130, 256, 16, "bf16", 1.0, False),
+        (77, 5, 5, "f32", 1.0, False),
+    ],
+)
+def test_routing_decision_is_bit_exact_given_logits(gpu, tokens, experts, top_k, dtype, scale, use_bias):
+    rng = np.random.default_rng(tokens * 1000 + experts)
+    logits = (rng.standard_normal((tokens, experts)) * 2.0).astype(np.float32)
+    if dtype == "bf16":
+        logits = O.bf16_round(logits)  # bf16 logits make exact score ties common
+    logits[0, :] = 0.0  # a fully tied row
+    if tokens > 2:
+        logits[1, :] = 40.0  # saturated: every score is exactly 1
+        logits[2, : experts // 2] = -100.0
+    bias = (rng.standard_normal(experts) * 0.3).astype(np.float32) if use_bias else None
+    want = O.router_from_logits(logits, bias, top_k, scale, dtype)
+    got = ops.router_from_logits(dev(logits, gpu), None if bias is None else dev(bias, gpu), top_k, scale,
+                                 dtype=torch.bfloat16 if dtype == "bf16" else torch.float32)
+    assert np.array_equal(host(got.scores), want.scores)
+    assert np.array_equal(host(got.expert_ids), want.expert_ids)
+    assert np.array_equal(host(got.weights), want.weights)
+    stats = O.router_stats(want.expert_ids, want.weights, experts)
+    assert np.array_equal(host(got.expert_counts), stats.expert_counts)
+    np.testing.assert_allclose(host(got.importance), stats.importance, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("case", ["router_order", "router_bias_scale"])
+def test_router_known_answers(gpu, kat, case):
+    c = kat[case]
+    bias = None if c["expert_bias"] is None else dev(np.asarray(c["expert_bias"], np.float32), gpu)
+    r = ops.router(dev(np.asarray(c["x"], np.float32), gpu), dev(np.asarray(c["w_router"], np.float32), gpu), bias,
+                   c["top_k"], c["route_scale"])
+    assert host(r.expert_ids).tolist() == c["expected"]["ids"]
+    np.testing.assert_allclose(host(r.weights), np.asarray(c["expected"]["weights"]), rtol=2e-6)
+    np.testing.assert_allclose(host(r.weights).sum(-1), c["asserted"]["weight_sum"], rtol=1e-6)
+
+
+def check_router_end_to_end(gpu, x, w, bias, top_k, scale, dtype):
+    """Logits within 1 ulp of the compute dtype; every routing difference must be
+    explained by a logit that differs; rows whose logits agree must agree bit for bit."""
+    want = O.router(x, w, bias, top_k, scale, dtype)
+    got = ops.router(dev(x, gpu, dtype), dev(w, gpu, dtype), None if bias is None else dev(bias, gpu), top_k, scale,
+                     return_logits=True)
+    g_logits = host(got.logits)
+    if dtype == "bf16":
+        assert np.array_equal(g_logits, O.bf16_round(g_logits))
+        ulp = np.maximum(np.abs(want.logits) * 2.0**-7, 1e-5)  # one bf16 ulp (fp32 sum error near zero)
+    else:
+        ulp = np.abs(want.logits) * 2e-5 + 2e-6
+    diff = np.abs(g_logits - want.logits)
+    assert np.all(diff <= ulp), f"logits differ by more than 1 ulp: {float(np.max(diff / ulp))}"
+    same_rows = np.all(g_logits == want.logits, axis=1)
+    print(f"[parity] router {dtype} T={x.shape[0]} E={w.shape[1]}: rows with identical logits "
+          f"{int(same_rows.sum())}/{x.shape[0]}, logits differing {int((diff > 0).sum())}", flush=True)
+    ids = host(got.expert_ids)
+    assert np.array_equal(ids[same_rows], want.expert_ids[same_rows])
+    assert np.array_equal(host(got.weights)[same_rows], want.weights[same_rows])
+    assert np.array_equal(host(got.scores)[same_rows], want.scores[same_rows])
+    # the kernel's decision is exactly the oracle's decision on the kernel's own logits
+    own = O.router_from_logits(g_logits, bias, top_k, scale, dtype)
+    assert np.array_equal(ids, own.expert_ids)
+    assert np.array_equal(host(got.weights), own.weights)
+    assert np.array_equal(host(got.scores), own.scores)
+    return ids
+
+
+@pytest.mark.parametrize(
+    "tokens,hidden,experts,top_k,dtype",
+    [(64, 32, 8, 2, "f32"), (257, 512, 8, 2, "f32"), (300, 1024, 16, 2, "bf16"), (1024, 2048, 64, 8, "bf16"),
+     (513, 2048, 128, 8, "bf16"), (100, 72, 24, 3, "bf16")],
+)
+def test_router_end_to_end(gpu, tokens, hidden, experts, top_k, dtype):
+    rng = np.random.default_rng(hidden + experts)
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    w = (rng.standard_normal((hidden, experts)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(experts) * 0.05).astype(np.float32)
+    check_router_end_to_end(gpu, x, w, bias, top_k, 1.0, dtype)
+
+
+# --------------------------------------------------------------------------
+# dispatch
+# --------------------------------------------------------------------------
+def check_dispatch(gpu, ids: np.ndarray, experts: int, x: np.ndarray | None, dtype: str = "f32"):
+    want = O.dispatch(ids, experts, None if x is None else O.cast_compute(x, dtype))
+    got = ops.dispatch(dev(ids, gpu), experts, None if x is None else dev(x, gpu, dtype))
+    assert np.array_equal(host(got.group_sizes), want.group_sizes)
+    assert np.array_equal(host(got.offsets), want.offsets)
+    assert np.array_equal(host(got.source_order), want.source_order)
+    assert np.array_equal(host(got.inverse), want.inverse)
+    if x is not None:
+        assert np.array_equal(host(got.packed_x), want.packed_x)
+    return got
+
+
+@pytest.mark.parametrize(
+    "tokens,top_k,experts,hidden,dtype",
+    [(1, 1, 1, 8, "f32"), (6, 2, 4, 3, "f32"), (511, 2, 8, 64, "bf16"), (512, 2, 8, 64, "bf16"), (513, 2, 8, 64, "bf16"),
+     (1000, 8, 64, 256, "bf16"), (4096, 8, 128, 40, "bf16"), (333, 3, 256, 7, "bf16"), (2048, 2, 16, 1024, "f32")],
+)
+def test_dispatch_is_bit_exact(gpu, tokens, top_k, experts, hidden, dtype):
+    rng = np.random.default_rng(tokens + experts)
+    ids = rng.integers(0, experts, size=(tokens, top_k)).astype(np.int32)
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    check_dispatch(gpu, ids, experts, x, dtype)
+
+
+def test_dispatch_reference_edge_patterns(gpu, kat):
+    c = kat["edge_patterns"]
+    x = np.asarray(c["x"], np.float32)
+    for name, p in c["patterns"].items():
+        ids = np.asarray(p["expert_ids"], np.int32)
+        got = check_dispatch(gpu, ids, c["num_experts"], x)
+        again = ops.dispatch(dev(ids, gpu), c["num_experts"], dev(x, gpu))
+        assert torch.equal(got.source_order, again.source_order) and torch.equal(got.packed_x, again.packed_x), name
+
+
+def test_dispatch_skewed_and_empty(gpu):
+    rng = np.random.default_rng(9)
+    ids = np.minimum(rng.zipf(1.3, size=(5000, 8)) - 1, 127).astype(np.int32)  # heavy skew, many empty experts
+    check_dispatch(gpu, ids, 128, None)
+    check_dispatch(gpu, np.zeros((3000, 4), np.int32), 64, rng.standard_normal((3000, 16)).astype(np.float32), "bf16")
+    empty = ops.dispatch(torch.zeros((0, 2), dtype=torch.int32, device=gpu), 4)
+    assert host(empty.group_sizes).tolist() == [0, 0, 0, 0] and host(empty.offsets).tolist() == [0, 0, 0, 0]
+
+
+# --------------------------------------------------------------------------
+# grouped SwiGLU, shared experts, combine
+# --------------------------------------------------------------------------
+def random_problem(seed, tokens, hidden, experts, top_k, inter, std=0.2):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    gate, up = (rng.standard_normal((experts, hidden, inter)).astype(np.float32) * std for _ in range(2))
+    down = rng.standard_normal((experts, inter, hidden)).astype(np.float32) * std
+    ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    w = rng.random((tokens, top_k)).astype(np.float32)
+    w = w / w.sum(-1, keepdims=True)
+    return x, gate, up, down, ids, w
+
+
+@pytest.mark.parametrize(
+    "tokens,hidden,experts,top_k,inter,dtype",
+    [(8, 3, 4, 2, 5, "f32"), (70, 32, 4, 2, 64, "f32"), (200, 512, 8, 2, 1024, "f32"),
+     (8, 3, 4, 2, 5, "bf16"), (300, 64, 6, 3, 96, "bf16"), (700, 1024, 16, 2, 2816, "bf16"),
+     (512, 2048, 64, 8, 1408, "bf16"), (64, 2048, 64, 8, 1408, "bf16"), (257, 200, 5, 2, 136, "bf16")],
+)
+def test_grouped_swiglu_matches_oracle(gpu, tokens, hidden, experts, top_k, inter, dtype):
+    std = 0.02 if hidden >= 512 else 0.2
+    x, gate, up, down, ids, _ = random_problem(tokens + inter, tokens, hidden, experts, top_k, inter, std)
+    d = O.dispatch(ids, experts, O.cast_compute(x, dtype))
+    want, _, _, want_act = O.grouped_swiglu(d.packed_x, gate, up, down, d.group_sizes, dtype, return_stages=True)
+    got, act = ops.grouped_swiglu(dev(d.packed_x, gpu, dtype), dev(gate, gpu, dtype), dev(up, gpu, dtype),
+                                  dev(down, gpu, dtype), dev(d.group_sizes, gpu), dev(d.offsets, gpu), return_act=True)
+    tag = f"grouped_swiglu {dtype} T={tokens} H={hidden} E={experts} K={top_k} I={inter}"
+    if dtype == "bf16":
+        assert report(tag + " act", host(act), want_act) <= BF16_MAX_REL
+        assert report(tag + " y", host(got), want) <= BF16_MAX_REL
+    else:
+        np.testing.assert_allclose(host(act), want_act, **F32_TOL)
+        np.testing.assert_allclose(host(got), want, **F32_TOL)
+
+
+def test_grouped_swiglu_empty_groups_and_single_expert(gpu):
+    rng = np.random.default_rng(21)
+    H, I, E = 64, 96, 8
+    x = rng.standard_normal((50, H)).astype(np.float32)
+    gate, up = (rng.standard_normal((E, H, I)).astype(np.float32) * 0.2 for _ in range(2))
+    down = rng.standard_normal((E, I, H)).astype(np.float32) * 0.2
+    sizes = np.array([0, 50, 0, 0, 0, 0, 0, 0], np.int32)  # every row on expert 1
+    offs = np.array([0, 0, 50, 50, 50, 50, 50, 50], np.int32)
+    got = ops.grouped_swiglu(dev(x, gpu, "bf16"), dev(gate, gpu, "bf16"), dev(up, gpu, "bf16"), dev(down, gpu, "bf16"),
+                             dev(sizes, gpu), dev(offs, gpu))
+    want = O.grouped_swiglu(O.bf16_round(x), gate, up, down, sizes, "bf16")
+    assert report("single live expert", host(got), want) <= BF16_MAX_REL
+    # against a plain matmul in float64 (the one-expert special case)
+    xb, gb, ub, db = (O.bf16_round(a).astype(np.float64) for a in (x, gate[1], up[1], down[1]))
+    g, u = xb @ gb, xb @ ub
+    dense = (g / (1 + np.exp(-g)) * u) @ db
+    assert rel_err(host(got), dense.astype(np.float32)) <= BF16_MAX_REL
+
+
+def test_expert_known_answers_fp32(gpu, kat):
+    for case in ("expert_swiglu_manual", "local_dispatcher", "dispatcher_equivalence"):
+        c = kat[case]
+        x, ids, w = (np.asarray(c[k], np.float32) for k in ("x", "expert_ids", "weights"))
+        ids = ids.astype(np.int32)
+        gate, up, down = (np.asarray(c[k], np.float32) for k in ("gate", "up", "down"))
+        d = ops.dispatch(dev(ids, gpu), gate.shape[0], dev(x, gpu))
+        y = ops.grouped_swiglu(d.packed_x, dev(gate, gpu), dev(up, gpu), dev(down, gpu), d.group_sizes, d.offsets)
+        out = ops.combine(y, d.inverse, dev(w, gpu))
+        np.testing.assert_allclose(host(out), np.asarray(c["expected"]["out"]), rtol=1e-5, atol=1e-5, err_msg=case)
+
+
+@pytest.mark.parametrize("group", ["edge_patterns", "profile_bench"])
+def test_edge_pattern_outputs_fp32(gpu, kat, group):
+    c = kat[group]
+    if group == "profile_bench":
+        E, H, I, S = c["num_experts"], c["hidden"], c["inter"], c["seq"]
+        gate = (np.arange(E * H * I, dtype=np.float32) / np.float32(4096.0)).reshape(E, H, I)
+        up = gate[..., ::-1].copy()
+        down = (np.arange(E * I * H, dtype=np.float32) / np.float32(4096.0)).reshape(E, I, H)
+        x = (np.arange(S * H, dtype=np.float32) / np.float32(512.0)).reshape(S, H)
+        w = np.full((S, c["top_k"]), 0.5, np.float32)
+    else:
+        gate, up, down, x, w = (np.asarray(c[k], np.float32) for k in ("gate", "up", "down", "x", "weights"))
+    for name, p in c["patterns"].items():
+        ids = np.asarray(p["expert_ids"], np.int32)
+
+        def run():
+            d = ops.dispatch(dev(ids, gpu), gate.shape[0], dev(x, gpu))
+            y = ops.grouped_swiglu(d.packed_x, dev(gate, gpu), dev(up, gpu), dev(down, gpu), d.group_sizes, d.offsets)
+            return ops.combine(y, d.inverse, dev(w, gpu))
+
+        first, second = run(), run()
+        np.testing.assert_allclose(host(first), np.asarray(p["expected_out"]), rtol=2e-5, atol=2e-5, err_msg=name)
+        assert torch.equal(first, second), name  # run twice: bit-identical
+
+
+@pytest.mark.parametrize("tokens,hidden,top_k,dtype,with_shared",
+                         [(9, 5, 3, "f32", True), (1000, 2048, 8, "bf16", True), (300, 1024, 2, "bf16", False),
+                          (77, 72, 4, "bf16", True), (64, 2048, 16, "bf16", False)])
+def test_combine_is_bit_exact(gpu, tokens, hidden, top_k, dtype, with_shared):
+    rng = np.random.default_rng(tokens)
+    packed_y = O.cast_compute(rng.standard_normal((tokens * top_k, hidden)).astype(np.float32), dtype)
+    inverse = rng.permutation(tokens * top_k).astype(np.int32)
+    w = O.cast_compute(rng.random((tokens, top_k)).astype(np.float32), dtype)
+    shared = O.cast_compute(rng.standard_normal((tokens, hidden)).astype(np.float32), dtype) if with_shared else None
+    want = O.combine(packed_y, inverse, w, dtype, shared)
+    got = ops.combine(dev(packed_y, gpu, dtype), dev(inverse, gpu), dev(w, gpu, dtype),
+                      None if shared is None else dev(shared, gpu, dtype))
+    assert np.array_equal(host(got), want)
+
+
+@pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16")])
+def test_shared_swiglu_matches_oracle(gpu, tokens, hidden, inter, dtype):
+    rng = np.random.default_rng(inter)
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    std = 0.02 if hidden >= 512 else 0.2
+    g, u = (rng.standard_normal((hidden, inter)).astype(np.float32) * std for _ in range(2))
+    dn = rng.standard_normal((inter, hidden)).astype(np.float32) * std
+    want = O.shared_swiglu(x, g, u, dn, dtype)
+    got = ops.shared_swiglu(dev(x, gpu, dtype), dev(g, gpu, dtype), dev(u, gpu, dtype), dev(dn, gpu, dtype))
+    if dtype == "bf16":
+        assert report(f"shared_swiglu T={tokens} H={hidden} Is={inter}", host(got), want) <= BF16_MAX_REL
+    else:
+        np.testing.assert_allclose(host(got), want, **F32_TOL)
+
+
+# --------------------------------------------------------------------------
+# statistics and the balance loss
+# --------------------------------------------------------------------------
+def test_router_stats_and_balance_loss(gpu, kat):
+    c = kat["balance_loss"]
+    loss = ops.sequence_balance_loss(dev(np.asarray(c["expert_ids"], np.int32), gpu),
+                                     dev(np.asarray(c["scores"], np.float32), gpu), top_k=c["top_k"])
+    assert abs(float(loss) - 0.975) < 1e-6
+    rng = np.random.default_rng(4)
+    B, S, E, K = 3, 50, 24, 4
+    scores = rng.random((B, S, E)).astype(np.float32)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(B * S)]).astype(np.int32).reshape(B, S, K)
+    want = O.sequence_balance_loss(ids, scores, K)
+    got = ops.sequence_balance_loss(dev(ids, gpu), dev(scores, gpu), top_k=K)
+    assert abs(float(got) - float(want)) <= 1e-5 * abs(float(want))
+    counts = np.array([5, 0, 9, 2, 0, 16], np.float32)
+    s = O.stats_from_counts(counts, counts)
+    got6 = host(ops.router_stats(dev(counts, gpu)))
+    np.testing.assert_allclose(
+        got6, [s.total_assignments, s.load_min, s.load_max, s.load_mean, s.max_vio, s.load_entropy], rtol=1e-6)
+
+
+# --------------------------------------------------------------------------
+# the whole layer through jtmoe_moe_forward
+# --------------------------------------------------------------------------
+def run_layer(gpu, inp, top_k, dtype):
+    cfg = inp["cfg"]
+    T = inp["x"].shape[0] * inp["x"].shape[1]
+    x2 = inp["x"].reshape(T, cfg["H"])
+    shared = None if inp["shared"] is None else tuple(dev(m, gpu, dtype) for m in inp["shared"])
+    got = ops.moe_forward(dev(x2, gpu, dtype), dev(inp["w_router"], gpu, dtype), dev(inp["expert_bias"], gpu),
+                          dev(inp["gate"], gpu, dtype), dev(inp["up"], gpu, dtype), dev(inp["down"], gpu, dtype),
+                          top_k, 1.0, shared=shared)
+    return x2, got
+
+
+def check_layer_against_oracle(gpu, inp, top_k, dtype, tag):
+    """Staged comparison: the oracle is evaluated on the kernel's own routing
+    (which test_router_end_to_end ties to the oracle's), so that one flipped
+    near-tie does not hide the numerical comparison of the expert outputs."""
+    x2, got = run_layer(gpu, inp, top_k, dtype)
+    E = inp["gate"].shape[0]
+    ids = host(got.expert_ids)
+    ref_route = O.router(x2, inp["w_router"], inp["expert_bias"], top_k, 1.0, dtype)
+    mism = int(np.sum(np.any(ids != ref_route.expert_ids, axis=1)))
+    print(f"[parity] {tag}: tokens routed differently from the oracle's own logits: {mism}/{x2.shape[0]}", flush=True)
+    assert mism <= max(1, x2.shape[0] // 500)
+    d = O.dispatch(ids, E, O.cast_compute(x2, dtype))
+    assert np.array_equal(host(got.group_sizes), d.group_sizes)
+    assert np.array_equal(host(got.offsets), d.offsets)
+    assert np.array_equal(host(got.source_order), d.source_order)
+    assert np.array_equal(host(got.inverse), d.inverse)
+    assert np.array_equal(host(got.expert_counts), d.group_sizes.astype(np.float32))
+    packed_y = O.grouped_swiglu(d.packed_x, inp["gate"], inp["up"], inp["down"], d.group_sizes, dtype)
+    shared_y = None if inp["shared"] is None else O.shared_swiglu(x2, *inp["shared"], dtype)
+    want = O.combine(packed_y, d.inverse, host(got.weights), dtype, shared_y)
+    stats = O.router_stats(ids, host(got.weights), E)
+    np.testing.assert_allclose(host(got.importance), stats.importance, rtol=1e-5, atol=1e-4)
+    y = host(got.y)
+    if dtype == "bf16":
+        assert report(tag, y, want) <= BF16_MAX_REL
+    else:
+        np.testing.assert_allclose(y, want, rtol=1e-4, atol=2e-5)
+    return got
+
+
+def test_layer_c1_fp32(gpu):
+    inp = O.make_inputs("C1", seed=0)
+    got = check_layer_against_oracle(gpu, inp, 2, "f32", "C1 fp32 T=2048 H=512 E=8 K=2 I=1024")
+    ref = O.router(inp["x"][0], inp["w_router"], inp["expert_bias"], 2, 1.0, "f32")
+    assert int(np.sum(np.any(host(got.expert_ids) != ref.expert_ids, axis=1))) == 0  # fp32: no near-ties flip
+
+
+def test_layer_c2_shape_bf16_sample(gpu):
+    inp = O.make_inputs("C2", seed=0, tokens=1024)
+    check_layer_against_oracle(gpu, inp, 2, "bf16", "C2 bf16 sample T=1024 H=1024 E=16 K=2 I=2816")
+
+
+def test_layer_c3_shape_bf16_sample_with_shared(gpu):
+    inp = O.make_inputs("C3", seed=0, tokens=768)
+    check_layer_against_oracle(gpu, inp, 8, "bf16", "C3 bf16 sample T=768 H=2048 E=64 K=8 I=1408 Ns=2")
+
+
+def test_layer_c4_skewed_bf16_sample(gpu):
+    inp = O.make_inputs("C4", seed=0, tokens=1024)
+    got = check_layer_against_oracle(gpu, inp, 8, "bf16", "C4 bf16 sample T=1024 H=2048 E=128 K=8 I=768 skew")
+    assert int((host(got.group_sizes) == 0).sum()) >= 6
+
+
+def test_layer_c5_decode_and_per_token_property(gpu):
+    inp = O.make_inputs("C5", seed=0)
+    got = check_layer_against_oracle(gpu, inp, 8, "bf16", "C5 bf16 T=64 H=2048 E=64 K=8 I=1408")
+    # a token's output does not depend on the rest of the batch
+    sub = dict(inp)
+    sub["x"] = inp["x"][10:23]
+    _, part = run_layer(gpu, sub, 8, "bf16")
+    assert torch.equal(part.expert_ids, got.expert_ids[10:23])
+    assert torch.equal(part.weights, got.weights[10:23])
+    assert rel_err(host(part.y), host(got.y[10:23])) <= 1e-2
+
+
+def test_layer_twice_is_bit_identical(gpu):
+    inp = O.make_inputs("C2", seed=1, tokens=512)
+    _, a = run_layer(gpu, inp, 2, "bf16")
+    a_y, a_ids, a_imp = a.y.clone(), a.expert_ids.clone(), a.importance.clone()
+    _, b = run_layer(gpu, inp, 2, "bf16")
+    assert torch.equal(a_y, b.y) and torch.equal(a_ids, b.expert_ids) and torch.equal(a_imp, b.importance)

@@ -1,0 +1,62 @@
+"""Host-layer contract: spec validation and the operators' refusal to run
+anywhere but on the GPU (there is no CPU path to fall back to)."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from research_amd import moe, ops
+from research_amd.errors import ContractError
+
+
+def test_spec_validation_follows_the_reference_contract():
+    ok = moe.TrinityMoeSpec(num_experts=8, top_k=2, expert_intermediate_size=64)
+    assert ok.balance.name == "none" and ok.route_scale == 1.0
+    assert moe.TrinityMoeSpec(4, 2, balance={"name": "smebu"}).balance.name == "smebu"
+    for kwargs in (
+        dict(num_experts=0, top_k=1),
+        dict(num_experts=4, top_k=5),
+        dict(num_experts=4, top_k=True),
+        dict(num_experts=4, top_k=2, expert_intermediate_size=0),
+        dict(num_experts=4, top_k=2, num_shared_experts=-1),
+        dict(num_experts=4, top_k=2, route_scale=0.0),
+        dict(num_experts=4, top_k=2, balance={"name": "aux"}),
+        dict(num_experts=4, top_k=2, balance={"name": "smebu", "sequence_aux_loss_weight": -1.0}),
+        dict(num_experts=4, top_k=2, balance=3),
+    ):
+        with pytest.raises(ContractError):
+            moe.TrinityMoeSpec(**kwargs)
+
+
+def test_router_constructor_checks():
+    for kw in (dict(num_experts=3, top_k=4), dict(num_experts=3, top_k=0), dict(num_experts=3, top_k=2, route_scale=0.0)):
+        with pytest.raises(ContractError):
+            moe.SigmoidTopKRouter(2, dtype=torch.float32, param_dtype=torch.float32, device="cpu", **kw)
+
+
+def test_layer_requires_resolved_intermediate_size():
+    with pytest.raises(ContractError, match="expert_intermediate_size"):
+        moe.SparseMoE(8, moe.TrinityMoeSpec(4, 2), device="cpu")
+
+
+def test_operators_refuse_cpu_tensors():
+    x = torch.zeros((4, 8))
+    w = torch.zeros((8, 4))
+    with pytest.raises(ContractError, match="GPU"):
+        ops.router(x, w, None, 2)
+    with pytest.raises(ContractError, match="GPU"):
+        ops.dispatch(torch.zeros((4, 2), dtype=torch.int32), 4)
+    with pytest.raises(ContractError, match="GPU"):
+        ops.combine(torch.zeros((8, 8)), torch.zeros(8, dtype=torch.int32), torch.zeros((4, 2)))
+    layer = moe.SparseMoE(8, moe.TrinityMoeSpec(4, 2, expert_intermediate_size=16), compute_dtype="float32", device="cpu")
+    with pytest.raises(ContractError, match="GPU"):
+        layer(torch.zeros((1, 4, 8)))
+    with pytest.raises(ContractError, match="one device"):
+        layer(torch.zeros((1, 4, 8)), execution=object())
+
+
+def test_dtype_names():
+    assert moe.dtype_from_name("bfloat16") is torch.bfloat16
+    with pytest.raises(ContractError):
+        moe.dtype_from_name("float16")
