@@ -10,52 +10,12 @@
 // are accumulated in fp32 on the matrix cores (v_mfma_f32_32x32x16_bf16 for
 // bf16, v_mfma_f32_32x32x2_f32 for fp32).
 #include "common.hpp"
+#include "grouped_gemm_fast.hpp"
+
+#include <mutex>
 
 namespace jtmoe {
 namespace {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
-
-// Row range of one m-tile.  Groups are the experts' contiguous row ranges; tile
-// `mt` counts m-tiles expert by expert (ceil(group_size / BM) each).
-struct TileRows {
-  int expert;
-  int row0;  // first packed row of the tile
-  int rows;  // valid rows in the tile (0 = no such tile)
-};
-
-__device__ __forceinline__ TileRows find_tile(int mt, int BM, const int32_t* __restrict__ group_sizes,
-                                              const int32_t* __restrict__ offsets, int E, int dense_rows) {
-  TileRows r;
-  r.expert = 0;
-  r.row0 = 0;
-  r.rows = 0;
-  if (group_sizes == nullptr) {
-    const int row0 = mt * BM;
-    if (row0 < dense_rows) {
-      r.row0 = row0;
-      r.rows = min(BM, dense_rows - row0);
-    }
-    return r;
-  }
-  int first = 0;
-  for (int e = 0; e < E; ++e) {
-    const int n = group_sizes[e];
-    const int tiles = (n + BM - 1) / BM;
-    if (mt < first + tiles) {
-      const int local = mt - first;
-      r.expert = e;
-      r.row0 = offsets[e] + local * BM;
-      r.rows = min(BM, n - local * BM);
-      return r;
-    }
-    first += tiles;
-  }
-  return r;
-}
-
-__device__ __forceinline__ float silu_fast(float g) { return g / (1.0f + __expf(-g)); }
 
 // ---------------------------------------------------------------------------
 // Generic kernel: any shape, any alignment, both dtypes.  64x64x32 tiles, four
@@ -102,7 +62,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(
 
   const int mt = blockIdx.x / ntiles_n;
   const int nt = blockIdx.x - mt * ntiles_n;
-  const TileRows tr = find_tile(mt, GBM, group_sizes, offsets, E, dense_rows);
+  const TileRows tr = find_tile_wave(mt, GBM, group_sizes, offsets, E, dense_rows);
   if (tr.rows <= 0) return;
   const int n0 = nt * GBN;
   const size_t wofs = (size_t)tr.expert * Kdim * N;
@@ -171,28 +131,67 @@ inline int64_t max_m_tiles(int64_t rows, int64_t groups, int BM) {
   return (rows + BM - 1) / BM + (groups < rows ? groups : rows);
 }
 
+template <typename T, bool kDual>
+int launch_generic(const void* a, const void* b0, const void* b1, void* c, const int32_t* group_sizes,
+                   const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream) {
+  const bool dense = group_sizes == nullptr;
+  const int64_t mtiles = dense ? (rows + GBM - 1) / GBM : max_m_tiles(rows, E, GBM);
+  const int64_t nt = (N + GBN - 1) / GBN;
+  if (mtiles * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
+  grouped_gemm_generic_kernel<T, kDual><<<(unsigned)(mtiles * nt), 256, 0, stream>>>(
+      static_cast<const T*>(a), static_cast<const T*>(b0), static_cast<const T*>(b1), static_cast<T*>(c), group_sizes,
+      offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)nt);
+  return JTMOE_OK;
+}
+
+template <typename Cfg>
+int launch_fast(const void* a, const void* b0, const void* b1, void* c, const int32_t* group_sizes,
+                const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream) {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  auto kernel = grouped_gemm_fast_kernel<Cfg>;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)Cfg::SMEM_BYTES);
+  });
+  if (attr_err != hipSuccess)
+    return fail(JTMOE_ELAUNCH, "grouped gemm: hipFuncSetAttribute: %s", hipGetErrorString(attr_err));
+  const bool dense = group_sizes == nullptr;
+  const int64_t mtiles = dense ? (rows + Cfg::BM - 1) / Cfg::BM : max_m_tiles(rows, E, Cfg::BM);
+  const int64_t nt = (N + Cfg::BN - 1) / Cfg::BN;
+  const int64_t grid = fast_gemm_grid(mtiles, nt);
+  if (grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
+  kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
+      static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
+      static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt);
+  return JTMOE_OK;
+}
+
+using GateUpCfg = FastGemmCfg<256, 128, 64, 4, 2, true>;
+using DownCfg = FastGemmCfg<256, 256, 64, 4, 2, false>;
+
+inline bool fast_ok(const void* a, const void* b0, const void* b1, const void* c, int64_t Kdim, int64_t N) {
+  return Kdim % 64 == 0 && N % 8 == 0 && Kdim * N < ((int64_t)1 << 30) && aligned16(a) && aligned16(b0) && (b1 == nullptr || aligned16(b1)) &&
+         aligned16(c);
+}
+
 template <typename T>
 int launch_pair(const void* x, const void* gate, const void* up, const void* down, const int32_t* group_sizes,
                 const int32_t* offsets, int64_t rows, int64_t H, int64_t I, int64_t E, void* act, void* y,
                 hipStream_t stream, int first_stage) {
-  const bool dense = group_sizes == nullptr;
-  const int64_t mtiles = dense ? (rows + GBM - 1) / GBM : max_m_tiles(rows, E, GBM);
-  if (mtiles == 0) return JTMOE_OK;
-  {
-    const int64_t nt = (I + GBN - 1) / GBN;
-    if (mtiles * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
-    grouped_gemm_generic_kernel<T, true><<<(unsigned)(mtiles * nt), 256, 0, stream>>>(
-        static_cast<const T*>(x), static_cast<const T*>(gate), static_cast<const T*>(up), static_cast<T*>(act),
-        group_sizes, offsets, (int)E, (int)rows, (int)H, (int)I, (int)nt);
-  }
+  if (rows == 0) return JTMOE_OK;
+  int rc;
+  if (Elem<T>::is_bf16 && fast_ok(x, gate, up, act, H, I))
+    rc = launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream);
+  else
+    rc = launch_generic<T, true>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream);
+  if (rc) return rc;
   stage_mark(first_stage, stream);
-  {
-    const int64_t nt = (H + GBN - 1) / GBN;
-    if (mtiles * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
-    grouped_gemm_generic_kernel<T, false><<<(unsigned)(mtiles * nt), 256, 0, stream>>>(
-        static_cast<const T*>(act), static_cast<const T*>(down), nullptr, static_cast<T*>(y), group_sizes, offsets,
-        (int)E, (int)rows, (int)I, (int)H, (int)nt);
-  }
+  if (Elem<T>::is_bf16 && fast_ok(act, down, nullptr, y, I, H))
+    rc = launch_fast<DownCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
+  else
+    rc = launch_generic<T, false>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
+  if (rc) return rc;
   stage_mark(first_stage + 1, stream);
   return check_launch("grouped gemm");
 }
