@@ -238,6 +238,134 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
                      router_scratch(ws, E));
 }
 
+// ---------------------------------------------------------------------------
+// bf16 projection on the matrix cores.  One workgroup = 64 tokens = 4 waves of 16
+// tokens; each wave owns all E columns of its tokens (NB = E/16 accumulator tiles of
+// v_mfma_f32_16x16x32_bf16).  x is read straight from HBM into MFMA operand
+// registers (each lane 32 contiguous bytes per 64-wide k chunk, whole 128-byte
+// lines per token row); the router matrix [H,E] is staged chunk by chunk through
+// LDS as it is stored and read with the transposing ds_read_b64_tr_b16.
+// Requires H % 64 == 0 and E in {16, 32, 64, 128, 256}.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+constexpr int kBufferFlags = 0x00020000;
+constexpr int kRouterKC = 64;  // k rows of the router matrix per LDS stage
+
+__host__ __device__ inline int router_w_stride(int E) { return E + 32; }  // elements; +64 B between k rows
+__host__ __device__ inline size_t router_mfma_smem_bytes(int E, int K) {
+  const size_t w = (size_t)2 * kRouterKC * router_w_stride(E) * 2;
+  const size_t ep = router_smem_bytes(E, K);
+  return w > ep ? w : ep;
+}
+
+template <int NB>
+__global__ __launch_bounds__(kRouterThreads) void router_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
+    int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
+    float* __restrict__ scores, float* __restrict__ logits_out, void* ws) {
+  constexpr int E = NB * 16;
+  constexpr int WS = E + 32;                      // LDS row stride of the staged matrix (elements)
+  constexpr int W_CHUNKS = kRouterKC * E / 8;     // 16-byte chunks per stage
+  constexpr int CW = (W_CHUNKS + kRouterThreads - 1) / kRouterThreads;
+  constexpr int CPR = E / 8;                      // chunks per k row
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  uint16_t* const Ws = reinterpret_cast<uint16_t*>(smem_raw);  // [2][kRouterKC][WS]; reused by the epilogue
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int t0 = blockIdx.x * kRouterTokens;
+  const int nrows = min(kRouterTokens, tokens - t0);
+
+  // x: lane (m = lane%16, kg = lane/16) holds k = chunk*64 + kg*16 + [0,16) of token t0 + wave*16 + m
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(x + (size_t)t0 * H), 0, nrows * H * 2, kBufferFlags);
+  const int x_voff = ((wave * 16 + (lane & 15)) * H + (lane >> 4) * 16) * 2;
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(w), 0, H * E * 2, kBufferFlags);
+
+  u32x4_t a_cur[2], a_nxt[2], w_reg[CW];
+  f32x4_t acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[nb][i] = 0.0f;
+
+#define JT_LOAD_W(k0)                                                                        \
+  _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                           \
+    const int c = tid + i * kRouterThreads;                                                  \
+    if (W_CHUNKS % kRouterThreads == 0 || c < W_CHUNKS)                                      \
+      w_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c * 16, (k0)*E * 2, 0);       \
+  }
+#define JT_STORE_W(stage)                                                                    \
+  _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                           \
+    const int c = tid + i * kRouterThreads;                                                  \
+    if (W_CHUNKS % kRouterThreads == 0 || c < W_CHUNKS) {                                    \
+      const int kr = c / CPR, nc = c - kr * CPR;                                             \
+      *reinterpret_cast<u32x4_t*>(Ws + ((stage)*kRouterKC + kr) * WS + nc * 8) = w_reg[i];   \
+    }                                                                                        \
+  }
+#define JT_LOAD_X(dst, k0)                                                                   \
+  {                                                                                          \
+    dst[0] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff, (k0)*2, 0);               \
+    dst[1] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff + 16, (k0)*2, 0);          \
+  }
+
+  // transposing read of this lane: 16-lane group kg = lane/16 reads rows kg*16 + 8*s + 4*h + i/4
+  const int w_lane = ((lane >> 4) * 16 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
+  const int nchunks = H / kRouterKC;
+  JT_LOAD_W(0);
+  JT_LOAD_X(a_cur, 0);
+  JT_STORE_W(0);
+  __syncthreads();
+  for (int kc = 0; kc < nchunks; ++kc) {
+    const int stage = kc & 1;
+    if (kc + 1 < nchunks) {
+      JT_LOAD_W((kc + 1) * kRouterKC);
+      JT_LOAD_X(a_nxt, (kc + 1) * kRouterKC);
+    }
+    const uint16_t* wbase = Ws + stage * kRouterKC * WS + w_lane;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_cur[s]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const uint16_t* p = wbase + s * 8 * WS + nb * 16;
+        const s16x4_t lo =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+        const s16x4_t hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
+        const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
+      }
+    }
+    if (kc + 1 < nchunks) {
+      JT_STORE_W(stage ^ 1);
+      a_cur[0] = a_nxt[0];
+      a_cur[1] = a_nxt[1];
+    }
+    __syncthreads();
+  }
+#undef JT_LOAD_W
+#undef JT_STORE_W
+#undef JT_LOAD_X
+
+  // logits (rounded to bf16, as the projection's output dtype) -> LDS tile; value i of lane l
+  // is token row 4*(l/16) + i, expert nb*16 + l%16
+  RouterSmem sm = router_smem(smem_raw, E, K);
+  const int stride = E + 1;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      sm.tile[(wave * 16 + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = round_to_bf16(acc[nb][i]);
+  __syncthreads();
+  router_epilogue<bf16_raw>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
+                            router_scratch(ws, E));
+}
+
 template <typename KernelT>
 int set_max_smem(KernelT kernel, size_t bytes) {
   if (bytes <= 64 * 1024) return JTMOE_OK;
@@ -252,17 +380,44 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
                   int64_t H, int64_t E, int64_t K, double route_scale, int32_t* ids, void* weights,
                   float* scores, float* counts, float* importance, float* logits_out, void* ws,
                   hipStream_t stream) {
-  const size_t smem = router_smem_bytes((int)E, (int)K);
-  if (smem > 160 * 1024) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
-  auto kernel = router_kernel<T, kFromLogits>;
-  int rc = set_max_smem(kernel, smem);
-  if (rc) return rc;
-  router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
-  if (tokens > 0) {
-    const int blocks = (int)((tokens + kRouterTokens - 1) / kRouterTokens);
-    kernel<<<blocks, kRouterThreads, smem, stream>>>(
-        static_cast<const T*>(x), static_cast<const T*>(w), logits_in, bias, (int)tokens, (int)H, (int)E, (int)K,
-        (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws);
+  const int blocks = (int)((tokens + kRouterTokens - 1) / kRouterTokens);
+  const bool mfma = Elem<T>::is_bf16 && !kFromLogits && H % kRouterKC == 0 && H * E < ((int64_t)1 << 30) &&
+                    (E == 16 || E == 32 || E == 64 || E == 128 || E == 256) && aligned16(x) && aligned16(w);
+  if (mfma) {
+    const size_t smem = router_mfma_smem_bytes((int)E, (int)K);
+    if (smem > 160 * 1024) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
+    router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
+    if (tokens > 0) {
+#define JT_ROUTER_CASE(NB)                                                                                   \
+  case NB * 16: {                                                                                            \
+    auto kernel = router_mfma_kernel<NB>;                                                                    \
+    int rc = set_max_smem(kernel, smem);                                                                     \
+    if (rc) return rc;                                                                                       \
+    kernel<<<blocks, kRouterThreads, smem, stream>>>(                                                        \
+        static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws);                   \
+    break;                                                                                                   \
+  }
+      switch ((int)E) {
+        JT_ROUTER_CASE(1)
+        JT_ROUTER_CASE(2)
+        JT_ROUTER_CASE(4)
+        JT_ROUTER_CASE(8)
+        JT_ROUTER_CASE(16)
+      }
+#undef JT_ROUTER_CASE
+    }
+  } else {
+    const size_t smem = router_smem_bytes((int)E, (int)K);
+    if (smem > 160 * 1024) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
+    auto kernel = router_kernel<T, kFromLogits>;
+    int rc = set_max_smem(kernel, smem);
+    if (rc) return rc;
+    router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
+    if (tokens > 0)
+      kernel<<<blocks, kRouterThreads, smem, stream>>>(
+          static_cast<const T*>(x), static_cast<const T*>(w), logits_in, bias, (int)tokens, (int)H, (int)E, (int)K,
+          (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws);
   }
   router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
   return check_launch("router");
