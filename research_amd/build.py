@@ -24,7 +24,10 @@ CACHE_SCHEMA_VERSION = 1
 MANIFEST_NAME = "manifest.json"
 LIBRARY_NAME = "libjtmoe.so"
 ARCH = "gfx950"
-SOURCE_FILES = ("api.hip", "router.hip", "dispatch.hip", "combine.hip", "grouped_gemm.hip", "common.hpp")
+SOURCE_FILES = (
+    "api.hip", "router.hip", "dispatch.hip", "combine.hip", "grouped_gemm.hip",
+    "common.hpp", "gemm_common.hpp", "grouped_gemm_dma.hpp",
+)
 
 
 def package_root() -> Path:

@@ -10,7 +10,7 @@
 // are accumulated in fp32 on the matrix cores (v_mfma_f32_32x32x16_bf16 for
 // bf16, v_mfma_f32_32x32x2_f32 for fp32).
 #include "common.hpp"
-#include "grouped_gemm_fast.hpp"
+#include "grouped_gemm_dma.hpp"
 
 #include <mutex>
 
@@ -149,7 +149,7 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
                 const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  auto kernel = grouped_gemm_fast_kernel<Cfg>;
+  auto kernel = grouped_gemm_dma_kernel<Cfg>;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)Cfg::SMEM_BYTES);
@@ -159,7 +159,7 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   const bool dense = group_sizes == nullptr;
   const int64_t mtiles = dense ? (rows + Cfg::BM - 1) / Cfg::BM : max_m_tiles(rows, E, Cfg::BM);
   const int64_t nt = (N + Cfg::BN - 1) / Cfg::BN;
-  const int64_t grid = fast_gemm_grid(mtiles, nt);
+  const int64_t grid = gemm_grid(mtiles, nt);
   if (grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
   kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
       static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
@@ -167,8 +167,10 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   return JTMOE_OK;
 }
 
-using GateUpCfg = FastGemmCfg<256, 128, 64, 4, 2, true>;
-using DownCfg = FastGemmCfg<256, 256, 64, 4, 2, false>;
+// 256 x 256 output tiles (gate and up share the A tile: 128 + 128 columns), 64-deep k steps,
+// two LDS stages, 8 waves
+using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16>;
+using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64>;
 
 inline bool fast_ok(const void* a, const void* b0, const void* b1, const void* c, int64_t Kdim, int64_t N) {
   return Kdim % 64 == 0 && N % 8 == 0 && Kdim * N < ((int64_t)1 << 30) && aligned16(a) && aligned16(b0) && (b1 == nullptr || aligned16(b1)) &&

@@ -1,0 +1,314 @@
+// Multi-stage bf16 grouped GEMM for gfx950 whose operand tiles are written into
+// LDS by the memory system itself (buffer_load_dwordx4 ... lds), not through
+// vector registers.
+//
+//   C[rows of group e, :] = A[rows of group e, :] @ B[e]          (kDual = false)
+//   C = silu(round(A @ B0[e])) * round(A @ B1[e])                  (kDual = true)
+//
+// A is [rows, K] row-major, B[e] is [K, N] row-major, as the expert matrices are
+// stored.  One wave-wide LDS load fills 1 KiB of LDS, lane i supplying bytes
+// [16 i, 16 i + 16); which 16 global bytes a lane fetches is free, so the tiles
+// are stored without padding and bank conflicts are avoided by permuting the
+// 16-byte chunks inside each row (an XOR swizzle applied to the *source* chunk):
+//   A tile [BM][BK]:        chunk c of row r sits in slot c ^ ((r / (16/CPR)) % CPR)
+//   B tile [BK][128] x NSUB: stored as 128-byte blocks of 4 k rows x 16 columns, so that
+//                            a 16-lane transposing read touches 128 contiguous bytes
+// A fragments are read with ds_read_b128, B fragments with the transposing
+// ds_read_b64_tr_b16 (lane i of a 16-lane group addresses row i/4, columns
+// 4*(i%4)..; lane j receives the four k values of its column j).
+//
+// NSTAGE tiles are in flight: iteration kt waits (s_waitcnt vmcnt) only for its own
+// tile, passes one barrier, re-arms the buffer that iteration kt-1 just released
+// and computes.  The loads are issued from inline assembly because the compiler
+// would otherwise drain every outstanding load before each LDS read.
+//
+// Requirements: K % BK == 0, N % 8 == 0, 16-byte aligned pointers, K*N*2 < 2^31.
+#pragma once
+
+#include "gemm_common.hpp"
+
+namespace jtmoe {
+
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+
+__device__ __forceinline__ unsigned lds_byte_addr(const void* p) {
+  return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+// 16 bytes per lane from a raw buffer straight into LDS at lds_base + lane*16.
+// Reads past the end of the buffer store zeros.
+__device__ __forceinline__ void buffer_load_lds16(i32x4_t rsrc, unsigned lds_base, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+               : "memory");
+}
+
+// fp32 -> bf16 by the hardware conversion (round to nearest even)
+__device__ __forceinline__ uint16_t bf16_bits_fast(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+__device__ __forceinline__ float bf16_round_fast(float f) { return (float)(__bf16)f; }
+// silu with the hardware exp2 and reciprocal (about 1 ulp each); results are rounded to bf16 anyway
+__device__ __forceinline__ float silu_rcp(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ i32x4_t make_rsrc(const void* base, int bytes) {
+  const unsigned long long p = (unsigned long long)base;
+  i32x4_t r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
+  r[1] = __builtin_amdgcn_readfirstlane((int)(unsigned)(p >> 32));
+  r[2] = __builtin_amdgcn_readfirstlane(bytes);
+  r[3] = kBufferFlags;
+  return r;
+}
+
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool kDual_, int NSTAGE_, int OPT_ = 16>
+struct DmaGemmCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NSTAGE = NSTAGE_;
+  // scheduling options: 16 = request the fragments of MFMA step kk+1 before issuing step kk,
+  // 32 = raise the wave priority around the MFMA burst, 64 = ask the scheduler to interleave
+  // one MFMA with up to three LDS reads
+  static constexpr int DBG = OPT_;
+  static constexpr bool kDual = kDual_;
+  static constexpr int BNE = kDual ? 2 * BN : BN;  // columns of the B tile in LDS
+  static constexpr int NSUB = BNE / 128;           // 128-column sub-tiles of B
+  static constexpr int NT = WAVES_M * WAVES_N * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BNE / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int TNO = kDual ? TN / 2 : TN;
+  static constexpr int WNO = TNO * 32;
+  static constexpr int CPRA = BK / 8;  // 16-byte chunks per A row
+  static constexpr int A_BYTES = BM * BK * 2;
+  static constexpr int BSUB_BYTES = BK * 256;
+  static constexpr int STAGE_BYTES = A_BYTES + NSUB * BSUB_BYTES;
+  static constexpr int A_LOADS = BM * CPRA / NT;   // per thread per stage
+  static constexpr int BSUB_LOADS = BK * 16 / NT;  // per thread per sub-tile per stage
+  static constexpr int LPS = A_LOADS + NSUB * BSUB_LOADS;
+  static constexpr int CS = WNO + 8;  // epilogue staging row stride (elements)
+  static constexpr size_t EPI_BYTES = (size_t)WAVES_M * WAVES_N * WM * CS * 2;
+  static constexpr size_t PIPE_BYTES = (size_t)NSTAGE * STAGE_BYTES;
+  static constexpr size_t SMEM_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
+  static constexpr int GROUP_M = 4;
+  static_assert(BNE % 128 == 0, "B tile is made of 128-column sub-tiles");
+  static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
+  static_assert((BM * CPRA) % NT == 0 && (BK * 16) % NT == 0, "tile must divide evenly over the threads");
+  static_assert((NT / CPRA) % 16 == 0 && NT % 64 == 0, "swizzle must not depend on the load index");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32x16 MFMAs");
+  static_assert(!kDual || (TN % 2 == 0 && BN == 128), "dual tiles: one sub-tile per matrix");
+  static_assert(NSTAGE >= 2 && (NSTAGE - 2) * LPS < 64, "vmcnt is a 6-bit counter");
+  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
+};
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
+    uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
+    int dense_rows, int Kdim, int N, int mtiles, int ntiles_n) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, NSTAGE = Cfg::NSTAGE;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
+  constexpr int CPRA = Cfg::CPRA;
+  constexpr bool kDual = Cfg::kDual;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+
+  // ---- block -> (m-tile, n-tile): consecutive workgroup ids go round-robin to the 8 XCDs,
+  // so give each XCD a contiguous range of the logical order, and walk that order in groups
+  // of GROUP_M m-tiles x all n-tiles so that neighbours share operand panels in their L2.
+  const int total = mtiles * ntiles_n;
+  const int per_xcd = (int)gridDim.x >> 3;
+  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (logical >= total) return;
+  const int group_span = Cfg::GROUP_M * ntiles_n;
+  const int group = logical / group_span;
+  const int in_group = logical - group * group_span;
+  const int gm = min(Cfg::GROUP_M, mtiles - group * Cfg::GROUP_M);
+  const int nt = in_group / gm;
+  const int mt = group * Cfg::GROUP_M + (in_group - nt * gm);
+
+  TileRows tr = find_tile_wave(mt, BM, group_sizes, offsets, E, dense_rows);
+  tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
+  tr.row0 = __builtin_amdgcn_readfirstlane(tr.row0);
+  tr.rows = __builtin_amdgcn_readfirstlane(tr.rows);
+  if (tr.rows <= 0) return;
+  const int n0 = nt * BN;
+  const size_t wofs = (size_t)tr.expert * Kdim * N;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WAVES_N, wn = wave - wm * Cfg::WAVES_N;
+
+  // ---- load plan ----
+  const i32x4_t a_rsrc = make_rsrc(A + (size_t)tr.row0 * Kdim, tr.rows * Kdim * 2);
+  i32x4_t b_rsrc[Cfg::NSUB];
+#pragma unroll
+  for (int u = 0; u < Cfg::NSUB; ++u)
+    b_rsrc[u] = make_rsrc((kDual && u == 1 ? B1 : B0) + wofs, Kdim * N * 2);
+  // A: slot s = j*NT + tid -> row s / CPRA, slot-in-row s % CPRA holds source chunk c
+  const int a_r = tid / CPRA, a_slot = tid - a_r * CPRA;
+  const int a_c = a_slot ^ ((a_r / (16 / CPRA)) % CPRA);
+  const int a_voff = (a_r * Kdim + a_c * 8) * 2;
+  // B sub-tile [BK][128]: stored as 128-byte blocks of 4 k rows x 16 columns, block (k/4, n/16) at
+  // index (k/4)*8 + n/16; slot s (16 bytes) -> block s/8, row (s/2)%4 of the block, half s%2
+  const int b_blk_id = tid >> 3;
+  const int b_k = (b_blk_id >> 3) * 4 + ((tid >> 1) & 3);
+  const int b_c = (b_blk_id & 7) * 2 + (tid & 1);
+  int b_voff[Cfg::NSUB];
+#pragma unroll
+  for (int u = 0; u < Cfg::NSUB; ++u) b_voff[u] = (b_k * N + n0 + (kDual ? 0 : u * 128) + b_c * 8) * 2;
+  const unsigned lds0 = lds_byte_addr(smem_raw);
+  const unsigned wave_lds = lds0 + wave * 1024;  // this wave's 1 KiB inside every NT*16-byte load round
+
+  auto issue = [&](int kt) {
+    const unsigned base = wave_lds + (kt % NSTAGE) * Cfg::STAGE_BYTES;
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int j = 0; j < Cfg::A_LOADS; ++j)
+      buffer_load_lds16(a_rsrc, base + j * NT * 16, a_voff + j * (NT / CPRA) * Kdim * 2, k0 * 2);
+#pragma unroll
+    for (int u = 0; u < Cfg::NSUB; ++u)
+#pragma unroll
+      for (int j = 0; j < Cfg::BSUB_LOADS; ++j)
+        buffer_load_lds16(b_rsrc[u], base + Cfg::A_BYTES + u * Cfg::BSUB_BYTES + j * NT * 16,
+                          b_voff[u] + j * (NT / 16) * N * 2, k0 * N * 2);
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
+
+  // ---- fragment addresses of this lane (bytes inside a stage) ----
+  const int a_row = wm * WM + (lane & 31);
+  const int a_sw = (a_row / (16 / CPRA)) % CPRA;
+  const int a_rowoff = a_row * (BK * 2);
+  // transposing read: the 16 lanes of a group read one whole 128-byte block, lane i its bytes
+  // [8 i, 8 i + 8) = row i/4, columns 4*(i%4)..; groups: column half (lane/16)%2, k half lane/32
+  const int b_laneoff = (lane & 15) * 8 + ((lane >> 4) & 1) * 128 + (lane >> 5) * (2 * 8 * 128);
+  int b_blk[TN];  // byte offset of column block jj: sub-tile base + its first 16-column block
+#pragma unroll
+  for (int jj = 0; jj < TN; ++jj) {
+    int col;  // first column of the block inside the BNE-wide tile
+    if (kDual)
+      col = (jj < TN / 2 ? 0 : BN) + wn * (WN / 2) + (jj % (TN / 2)) * 32;
+    else
+      col = wn * WN + jj * 32;
+    const int u = col >> 7, nblk = (col & 127) >> 4;
+    b_blk[jj] = Cfg::A_BYTES + u * Cfg::BSUB_BYTES + nblk * 128;
+  }
+
+  auto load_frags = [&](const unsigned char* st, int kk, bf16x8_t* af, bf16x8_t* bf) {
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi)
+      af[mi] = *reinterpret_cast<const bf16x8_t*>(st + a_rowoff + mi * 32 * BK * 2 +
+                                                  (((kk * 2 + (lane >> 5)) ^ a_sw) << 4));
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj) {
+      const unsigned char* p = st + b_blk[jj] + b_laneoff + kk * (4 * 8 * 128);
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+      const s16x4_t hi =
+          __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 8 * 128));
+      const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      bf[jj] = __builtin_bit_cast(bf16x8_t, both);
+    }
+  };
+
+  const int nk = Kdim / BK;
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s)
+    if (s < nk) issue(s);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    if (kt + NSTAGE - 2 < nk)
+      wait_vmcnt<(NSTAGE - 2) * Cfg::LPS>();
+    else
+      wait_vmcnt<0>();
+    __syncthreads();
+    if (kt + NSTAGE - 1 < nk) issue(kt + NSTAGE - 1);
+    const unsigned char* st = smem_raw + (kt % NSTAGE) * Cfg::STAGE_BYTES;
+    if (Cfg::DBG & 16) {
+      // fragments of step kk+1 are requested before the MFMAs of step kk are issued
+      bf16x8_t af[2][TM], bf[2][TN];
+      load_frags(st, 0, af[0], bf[0]);
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+        if (Cfg::DBG & 32) __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+          for (int jj = 0; jj < TN; ++jj)
+            acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
+        if (Cfg::DBG & 32) __builtin_amdgcn_s_setprio(0);
+        if (Cfg::DBG & 64) {
+          // interleave: one MFMA, then up to three LDS reads, repeated
+#pragma unroll
+          for (int g = 0; g < TM * TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        bf16x8_t af[TM], bf[TN];
+        load_frags(st, kk, af, bf);
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+          for (int jj = 0; jj < TN; ++jj)
+            acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bf[jj], acc[mi][jj], 0, 0, 0);
+      }
+    }
+  }
+  wait_vmcnt<0>();
+  __syncthreads();  // every wave is done reading the tiles: LDS becomes the output staging area
+
+  // ---- epilogue ----
+  // Value i of lane l in a 32x32 accumulator is row 8*(i/4) + 4*(l/32) + i%4, column l%32: a
+  // lane holds single elements of many rows.  Each wave parks its WM x WNO block of results
+  // in its own slice of the idle LDS and streams it out row by row with 16-byte stores.
+  constexpr int TNO = Cfg::TNO, WNO = Cfg::WNO, CS = Cfg::CS;
+  uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
+#pragma unroll
+  for (int mi = 0; mi < TM; ++mi) {
+#pragma unroll
+    for (int jj = 0; jj < TNO; ++jj) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+        float v;
+        if (kDual) {
+          const float g = bf16_round_fast(acc[mi][jj][i]);
+          const float u = bf16_round_fast(acc[mi][jj + TN / 2][i]);
+          v = silu_rcp(g) * u;
+        } else {
+          v = acc[mi][jj][i];
+        }
+        cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(v);
+      }
+    }
+  }
+  constexpr int CPR_OUT = WNO / 8;
+  constexpr int OUT_CHUNKS = WM * CPR_OUT;
+  const int col0 = n0 + wn * WNO;
+  const int row_base = wm * WM;
+#pragma unroll
+  for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
+    const int c = lane + j * 64;
+    const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
+    const int col = col0 + ch * 8;
+    if (row_base + r < tr.rows && col < N)
+      *reinterpret_cast<u32x4_t*>(C + (size_t)(tr.row0 + row_base + r) * N + col) = v;
+  }
+}
+
+}  // namespace jtmoe
