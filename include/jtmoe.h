@@ -120,6 +120,22 @@ int jtmoe_grouped_swiglu(const void* packed_x, const void* gate, const void* up,
                          void* act, void* packed_y, void* stream);
 
 /*
+ * Grouped SwiGLU with the row gather fused in.  Replaces sorted_x = flat_x[source_order]
+ * (moe.py:583, 595) together with the three ragged_dot calls (moe.py:638-641): packed row j is
+ * fetched from x[source_order[j] / K] while the GEMM loads its tiles, so packed_x is never
+ * materialised.  Same results as jtmoe_dispatch(..., x, packed_x) followed by
+ * jtmoe_grouped_swiglu.  Only for shapes jtmoe_grouped_swiglu_gather_supported() accepts
+ * (bf16, H and I multiples of 64); otherwise JTMOE_EUNSUPPORTED.
+ *   x [T,H] dtype; source_order [T*K] i32; others as jtmoe_grouped_swiglu.
+ */
+int jtmoe_grouped_swiglu_gather_supported(int64_t T, int64_t H, int64_t I, int dtype);
+int jtmoe_grouped_swiglu_gather(const void* x, const int32_t* source_order,
+                                const void* gate, const void* up, const void* down,
+                                const int32_t* group_sizes, const int32_t* offsets,
+                                int64_t T, int64_t K, int64_t H, int64_t I, int64_t E, int dtype,
+                                void* act, void* packed_y, void* stream);
+
+/*
  * Shared experts.  Replaces SharedSwiGLU.__call__ (moe.py:361-364) on one device
  * (execution.py:186-187, 199-200): one dense SwiGLU of width Is = I*num_shared.
  *   x [T,H]; gate, up [H,Is]; down [Is,H]; act [T,Is] workspace; out shared_y [T,H].

@@ -44,6 +44,11 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr],
     ),
+    "jtmoe_grouped_swiglu_gather_supported": (c_int, [c_i64, c_i64, c_i64, c_int]),
+    "jtmoe_grouped_swiglu_gather": (
+        c_int,
+        [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr],
+    ),
     "jtmoe_shared_swiglu": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr]),
     "jtmoe_combine": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr]),
     "jtmoe_router_stats": (c_int, [c_ptr, c_i64, c_ptr, c_ptr]),

@@ -267,11 +267,20 @@ extern "C" int jtmoe_moe_forward(const void* x, const void* w_router, const floa
                         expert_counts, importance, nullptr, w.router, w.router_bytes, stream);
   if (rc) return rc;
   stage_mark(kStageRouter, as_stream(stream));
-  rc = jtmoe_dispatch(expert_ids, T > 0 ? x : nullptr, T, H, E, K, dtype, group_sizes, offsets, source_order,
-                      inverse, w.packed_x, w.dispatch, w.dispatch_bytes, stream);
+  // where the GEMM can apply the permutation while it fetches its A tiles, the permuted copy of
+  // x is never written: dispatch then only computes the histogram, offsets and permutation
+  const bool gather = T > 0 && jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) &&
+                      (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(gate) & 15u) == 0 &&
+                      (reinterpret_cast<uintptr_t>(up) & 15u) == 0 && (reinterpret_cast<uintptr_t>(down) & 15u) == 0;
+  rc = jtmoe_dispatch(expert_ids, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes, offsets,
+                      source_order, inverse, w.packed_x, w.dispatch, w.dispatch_bytes, stream);
   if (rc) return rc;
-  rc = jtmoe_grouped_swiglu(w.packed_x, gate, up, down, group_sizes, offsets, T * K, H, I, E, dtype, w.act,
-                            w.packed_y, stream);
+  if (gather)
+    rc = jtmoe_grouped_swiglu_gather(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
+                                     w.act, w.packed_y, stream);
+  else
+    rc = jtmoe_grouped_swiglu(w.packed_x, gate, up, down, group_sizes, offsets, T * K, H, I, E, dtype, w.act,
+                              w.packed_y, stream);
   if (rc) return rc;
   if (Is > 0) {
     rc = jtmoe_shared_swiglu(x, shared_gate, shared_up, shared_down, T, H, Is, dtype, w.shared_act, w.shared_y,

@@ -146,7 +146,8 @@ int launch_generic(const void* a, const void* b0, const void* b1, void* c, const
 
 template <typename Cfg>
 int launch_fast(const void* a, const void* b0, const void* b1, void* c, const int32_t* group_sizes,
-                const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream) {
+                const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream,
+                const int32_t* row_map = nullptr, int row_div = 1, int64_t a_rows = 0) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   auto kernel = grouped_gemm_dma_kernel<Cfg>;
@@ -163,7 +164,8 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   if (grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
   kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
       static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
-      static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt);
+      static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,
+      row_map, row_div, (int)a_rows);
   return JTMOE_OK;
 }
 
@@ -180,11 +182,15 @@ inline bool fast_ok(const void* a, const void* b0, const void* b1, const void* c
 template <typename T>
 int launch_pair(const void* x, const void* gate, const void* up, const void* down, const int32_t* group_sizes,
                 const int32_t* offsets, int64_t rows, int64_t H, int64_t I, int64_t E, void* act, void* y,
-                hipStream_t stream, int first_stage) {
+                hipStream_t stream, int first_stage, const int32_t* row_map = nullptr, int row_div = 1,
+                int64_t x_rows = 0) {
   if (rows == 0) return JTMOE_OK;
   int rc;
   if (Elem<T>::is_bf16 && fast_ok(x, gate, up, act, H, I))
-    rc = launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream);
+    rc = launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map, row_div,
+                                x_rows);
+  else if (row_map != nullptr)
+    return fail(JTMOE_EUNSUPPORTED, "grouped_swiglu_gather: shape or alignment outside the gather-on-load path");
   else
     rc = launch_generic<T, true>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream);
   if (rc) return rc;
@@ -239,4 +245,32 @@ extern "C" int jtmoe_shared_swiglu(const void* x, const void* gate, const void* 
   if (dtype == JTMOE_BF16)
     return launch_pair<bf16_raw>(x, gate, up, down, nullptr, nullptr, T, H, Is, 1, act, shared_y, s, kStageSharedGateUp);
   return launch_pair<float>(x, gate, up, down, nullptr, nullptr, T, H, Is, 1, act, shared_y, s, kStageSharedGateUp);
+}
+
+extern "C" int jtmoe_grouped_swiglu_gather_supported(int64_t T, int64_t H, int64_t I, int dtype) {
+  return dtype == JTMOE_BF16 && H % 64 == 0 && I % 64 == 0 && H * I < ((int64_t)1 << 30) &&
+         T * H < ((int64_t)1 << 29);
+}
+
+extern "C" int jtmoe_grouped_swiglu_gather(const void* x, const int32_t* source_order, const void* gate,
+                                           const void* up, const void* down, const int32_t* group_sizes,
+                                           const int32_t* offsets, int64_t T, int64_t K, int64_t H, int64_t I,
+                                           int64_t E, int dtype, void* act, void* packed_y, void* stream) {
+  clear_error();
+  JT_REQUIRE(T >= 0 && K > 0 && T * K < ((int64_t)1 << 31), "grouped_swiglu_gather: T=%lld K=%lld out of range",
+             (long long)T, (long long)K);
+  const int64_t A = T * K;
+  int rc = validate_gemm("grouped_swiglu_gather", A, H, I, E, dtype);
+  if (rc) return rc;
+  if (E > JTMOE_MAX_EXPERTS)
+    return fail(JTMOE_EUNSUPPORTED, "grouped_swiglu_gather: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  if (A == 0) return JTMOE_OK;
+  JT_REQUIRE(x && source_order && gate && up && down && group_sizes && offsets && act && packed_y,
+             "grouped_swiglu_gather: null pointer argument");
+  if (!jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) || !aligned16(x))
+    return fail(JTMOE_EUNSUPPORTED,
+                "grouped_swiglu_gather: needs bf16, H and I multiples of 64 and 16-byte aligned rows "
+                "(use jtmoe_dispatch + jtmoe_grouped_swiglu otherwise)");
+  return launch_pair<bf16_raw>(x, gate, up, down, group_sizes, offsets, A, H, I, E, act, packed_y, as_stream(stream),
+                               kStageGateUp, source_order, (int)K, T);
 }

@@ -108,7 +108,8 @@ template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
     uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
-    int dense_rows, int Kdim, int N, int mtiles, int ntiles_n) {
+    int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
+    int a_rows) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, NSTAGE = Cfg::NSTAGE;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   constexpr int CPRA = Cfg::CPRA;
@@ -142,15 +143,30 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   const int wm = wave / Cfg::WAVES_N, wn = wave - wm * Cfg::WAVES_N;
 
   // ---- load plan ----
-  const i32x4_t a_rsrc = make_rsrc(A + (size_t)tr.row0 * Kdim, tr.rows * Kdim * 2);
   i32x4_t b_rsrc[Cfg::NSUB];
 #pragma unroll
   for (int u = 0; u < Cfg::NSUB; ++u)
     b_rsrc[u] = make_rsrc((kDual && u == 1 ? B1 : B0) + wofs, Kdim * N * 2);
+  // Without a row map, tile row r is row tr.row0 + r of A.  With one (gather on load), it is row
+  // row_map[tr.row0 + r] / row_div of A: the expert-major permutation is applied while the tile is
+  // fetched, so the permuted copy of the activations never exists in memory.
+  const bool gather = row_map != nullptr;
+  const i32x4_t a_rsrc = gather ? make_rsrc(A, a_rows * Kdim * 2)
+                                : make_rsrc(A + (size_t)tr.row0 * Kdim, tr.rows * Kdim * 2);
   // A: slot s = j*NT + tid -> row s / CPRA, slot-in-row s % CPRA holds source chunk c
   const int a_r = tid / CPRA, a_slot = tid - a_r * CPRA;
   const int a_c = a_slot ^ ((a_r / (16 / CPRA)) % CPRA);
-  const int a_voff = (a_r * Kdim + a_c * 8) * 2;
+  int a_voff[Cfg::A_LOADS];
+#pragma unroll
+  for (int j = 0; j < Cfg::A_LOADS; ++j) {
+    const int r = a_r + j * (NT / CPRA);
+    if (gather) {
+      // rows past the end of the group get an offset beyond the buffer: they read as zeros
+      a_voff[j] = r < tr.rows ? ((row_map[tr.row0 + r] / row_div) * Kdim + a_c * 8) * 2 : 0x70000000;
+    } else {
+      a_voff[j] = (r * Kdim + a_c * 8) * 2;
+    }
+  }
   // B sub-tile [BK][128]: stored as 128-byte blocks of 4 k rows x 16 columns, block (k/4, n/16) at
   // index (k/4)*8 + n/16; slot s (16 bytes) -> block s/8, row (s/2)%4 of the block, half s%2
   const int b_blk_id = tid >> 3;
@@ -167,7 +183,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     const int k0 = kt * BK;
 #pragma unroll
     for (int j = 0; j < Cfg::A_LOADS; ++j)
-      buffer_load_lds16(a_rsrc, base + j * NT * 16, a_voff + j * (NT / CPRA) * Kdim * 2, k0 * 2);
+      buffer_load_lds16(a_rsrc, base + j * NT * 16, a_voff[j], k0 * 2);
 #pragma unroll
     for (int u = 0; u < Cfg::NSUB; ++u)
 #pragma unroll

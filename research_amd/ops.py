@@ -238,6 +238,41 @@ def grouped_swiglu(
     return (packed_y, act) if return_act else packed_y
 
 
+def grouped_swiglu_gather(
+    x: torch.Tensor,
+    source_order: torch.Tensor,
+    top_k: int,
+    gate: torch.Tensor,
+    up: torch.Tensor,
+    down: torch.Tensor,
+    group_sizes: torch.Tensor,
+    offsets: torch.Tensor,
+) -> torch.Tensor:
+    """x [T,H] and the permutation -> packed_y [T*K,H] without materialising packed_x."""
+    _check(x, "x")
+    if x.dim() != 2:
+        raise ContractError(f"x must have shape [tokens, hidden], got {list(x.shape)}")
+    tokens, hidden = x.shape
+    _check(gate, "gate", x.dtype)
+    if gate.dim() != 3 or gate.shape[1] != hidden:
+        raise ContractError(f"expert gate matrix must have shape [experts, {hidden}, inter], got {list(gate.shape)}")
+    experts, _, inter = gate.shape
+    _check(up, "up", x.dtype, (experts, hidden, inter))
+    _check(down, "down", x.dtype, (experts, inter, hidden))
+    _check(source_order, "source_order", torch.int32, (tokens * top_k,))
+    _check(group_sizes, "group_sizes", torch.int32, (experts,))
+    _check(offsets, "offsets", torch.int32, (experts,))
+    dev = x.device
+    act = torch.empty((tokens * top_k, inter), dtype=x.dtype, device=dev)
+    packed_y = torch.empty((tokens * top_k, hidden), dtype=x.dtype, device=dev)
+    status = _lib().jtmoe_grouped_swiglu_gather(
+        _ptr(x), _ptr(source_order), _ptr(gate), _ptr(up), _ptr(down), _ptr(group_sizes), _ptr(offsets),
+        tokens, top_k, hidden, inter, experts, _code(x.dtype), _ptr(act), _ptr(packed_y), _stream(dev),
+    )
+    _raise(status, "jtmoe_grouped_swiglu_gather")
+    return packed_y
+
+
 def shared_swiglu(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
     """x [T,H]; gate, up [H,Is]; down [Is,H] -> [T,H]."""
     _check(x, "x")

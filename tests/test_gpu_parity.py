@@ -234,6 +234,31 @@ def test_grouped_swiglu_empty_groups_and_single_expert(gpu):
     assert rel_err(host(got), dense.astype(np.float32)) <= BF16_MAX_REL
 
 
+@pytest.mark.parametrize("tokens,hidden,experts,top_k,inter", [(700, 1024, 16, 2, 2816), (300, 2048, 64, 8, 1408),
+                                                               (64, 2048, 64, 8, 1408), (513, 128, 5, 3, 192)])
+def test_gather_on_load_equals_explicit_dispatch(gpu, tokens, hidden, experts, top_k, inter):
+    """jtmoe_grouped_swiglu_gather == jtmoe_dispatch (row copy) + jtmoe_grouped_swiglu, bit for bit."""
+    x, gate, up, down, ids, _ = random_problem(tokens, tokens, hidden, experts, top_k, inter, 0.03)
+    ids[: tokens // 3] = ids[0]  # skew: a third of the tokens share one expert set
+    xd, gd, ud, dd = (dev(a, gpu, "bf16") for a in (x, gate, up, down))
+    d = ops.dispatch(dev(ids, gpu), experts, xd)
+    explicit = ops.grouped_swiglu(d.packed_x, gd, ud, dd, d.group_sizes, d.offsets)
+    fused = ops.grouped_swiglu_gather(xd, d.source_order, top_k, gd, ud, dd, d.group_sizes, d.offsets)
+    assert torch.equal(explicit, fused)
+    want = O.grouped_swiglu(host(d.packed_x), gate, up, down, host(d.group_sizes), "bf16")
+    assert report(f"gather-on-load T={tokens} H={hidden} E={experts}", host(fused), want) <= BF16_MAX_REL
+
+
+def test_gather_on_load_refuses_unsupported_shapes(gpu):
+    from research_amd.errors import ContractError
+
+    x, gate, up, down, ids, _ = random_problem(3, 40, 72, 4, 2, 40)
+    xd, gd, ud, dd = (dev(a, gpu, "bf16") for a in (x, gate, up, down))
+    d = ops.dispatch(dev(ids, gpu), 4, xd)
+    with pytest.raises(ContractError, match="multiples of 64"):
+        ops.grouped_swiglu_gather(xd, d.source_order, 2, gd, ud, dd, d.group_sizes, d.offsets)
+
+
 def test_expert_known_answers_fp32(gpu, kat):
     for case in ("expert_swiglu_manual", "local_dispatcher", "dispatcher_equivalence"):
         c = kat[case]
