@@ -50,6 +50,18 @@ def algorithmic_work(cfg: dict) -> dict:
     )
 
 
+def measured_traffic(config: str, kernel: str):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc summary (None if absent).
+
+    bench.py cannot read hardware counters itself; profiles/hbm_traffic.json holds the scaled
+    FETCH_SIZE + WRITE_SIZE figures of the same command, and names the command that produced them."""
+    path = ROOT / "profiles" / "hbm_traffic.json"
+    try:
+        return json.loads(path.read_text())[config][kernel]["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def cpu_baseline(name: str, sample_tokens: int) -> dict:
     """The oracle (a NumPy port of the reference layer) timed on the host cores,
     on the first `sample_tokens` tokens of the same seeded workload."""
@@ -160,6 +172,42 @@ def main() -> int:
     stage_ms = {name: (sum(v) / len(v) if v else 0.0) for name, v in zip(_ffi.STAGE_NAMES, per_stage)}
     group_sizes = result.group_sizes.cpu().tolist()
 
+    # The fused layer applies the permutation inside the GEMM's tile loads, so its dispatch stage
+    # moves no rows.  The stand-alone dispatch entry point (histogram + scan + rank + row scatter
+    # into packed_x) is what a caller of the stage API runs: time it on the same routing.
+    def time_call(fn, iters):
+        for _ in range(3):
+            fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end) / iters
+
+    lib = _ffi.load_library()
+    A_rows = T * cfg["K"]
+    ids_fixed = result.expert_ids.clone()
+    d_sizes = torch.empty((cfg["E"],), dtype=torch.int32, device=dev)
+    d_offs = torch.empty_like(d_sizes)
+    d_order = torch.empty((A_rows,), dtype=torch.int32, device=dev)
+    d_inv = torch.empty_like(d_order)
+    d_packed = torch.empty((A_rows, cfg["H"]), dtype=tdtype, device=dev)
+    d_ws = torch.empty((lib.jtmoe_dispatch_workspace_bytes(A_rows, cfg["E"]),), dtype=torch.uint8, device=dev)
+    code = _ffi.JTMOE_BF16 if cfg["dtype"] == "bf16" else _ffi.JTMOE_F32
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def dispatch_call(with_rows):
+        rc = lib.jtmoe_dispatch(ids_fixed.data_ptr(), x.data_ptr() if with_rows else None, T, cfg["H"], cfg["E"],
+                                cfg["K"], code, d_sizes.data_ptr(), d_offs.data_ptr(), d_order.data_ptr(),
+                                d_inv.data_ptr(), d_packed.data_ptr(), d_ws.data_ptr(), d_ws.numel(), stream)
+        assert rc == 0, _ffi.last_error(lib)
+
+    dispatch_ms = time_call(lambda: dispatch_call(True), args.steps)
+    dispatch_meta_ms = time_call(lambda: dispatch_call(False), args.steps)
+    del d_packed
+
     work = algorithmic_work(cfg)
     peak = MFMA_BF16_PEAK_TFLOPS if cfg["dtype"] == "bf16" else MFMA_F32_PEAK_TFLOPS
 
@@ -177,20 +225,21 @@ def main() -> int:
         peak=peak,
         unit="TFLOP/s",
         frac=gate_up_tf / peak,
-        traffic=None,
+        traffic=measured_traffic(args.config, "gate_up"),
         avg_launch_ms=stage_ms["gate_up"],
         flops_per_launch=work["gate_up_flops"],
     )
-    dispatch_ms = stage_ms["dispatch_meta"] + stage_ms["dispatch_rows"]
     stages = dict(
         ms=stage_ms,
+        standalone_dispatch_ms=dispatch_ms,
+        standalone_dispatch_meta_ms=dispatch_meta_ms,
         grouped_gemm_mfma_util=tflops(work["gate_up_flops"] + work["down_flops"], stage_ms["gate_up"] + stage_ms["down"]) / peak,
         down_tflops=tflops(work["down_flops"], stage_ms["down"]),
         shared_tflops=tflops(work["shared_gate_up_flops"] + work["shared_down_flops"],
                              stage_ms["shared_gate_up"] + stage_ms["shared_down"]),
         router_gbs=gbs(work["router_bytes"], stage_ms["router"]),
         dispatch_gbs=gbs(work["dispatch_bytes"], dispatch_ms),
-        dispatch_rows_gbs=gbs(work["dispatch_rows_bytes"], stage_ms["dispatch_rows"]),
+        dispatch_rows_gbs=gbs(work["dispatch_rows_bytes"], max(dispatch_ms - dispatch_meta_ms, 1e-6)),
         combine_gbs=gbs(work["combine_bytes"], stage_ms["combine"]),
         hbm_peak_gbs=HBM_PEAK_GBS,
     )

@@ -11,8 +11,6 @@
 namespace jtmoe {
 namespace {
 
-constexpr int kMaxK = JTMOE_MAX_TOP_K;
-
 // 8 bf16 values per 16-byte vector
 __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -23,14 +21,28 @@ __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
   }
 }
 
-__device__ __forceinline__ uint4 pack8(const float* f) {
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+
+// fp32 -> bf16 -> fp32 with the hardware conversion (round to nearest even, same result as the
+// integer formula of f32_to_bf16_bits for every finite value)
+__device__ __forceinline__ float round_bf16_hw(float f) { return (float)(__bf16)f; }
+
+__device__ __forceinline__ uint4 pack8_hw(const float* f) {
   uint32_t w[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(f[2 * i]) | (f32_to_bf16_bits(f[2 * i + 1]) << 16);
+  for (int i = 0; i < 4; ++i) {
+    f32x2_t v = {f[2 * i], f[2 * i + 1]};
+    w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+  }
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// bf16, rows a multiple of 8 elements, 16-byte aligned: one wave streams rows
+// bf16, rows a multiple of 8 elements, 16-byte aligned.  One wave per token; a lane owns NV
+// 16-byte vectors of the row and requests them from all K source rows before it starts adding,
+// so K*NV independent loads are in flight per lane.  KT = K when K is one of the unrolled
+// values, 0 for a run-time loop.
+template <int NV, int KT>
 __global__ __launch_bounds__(256) void combine_bf16_vec_kernel(const uint4* __restrict__ packed_y,
                                                                const int32_t* __restrict__ inverse,
                                                                const uint16_t* __restrict__ weights,
@@ -39,40 +51,73 @@ __global__ __launch_bounds__(256) void combine_bf16_vec_kernel(const uint4* __re
 #pragma clang fp contract(off)
   const int t = blockIdx.x * blockDim.y + threadIdx.y;
   if (t >= tokens) return;
-  int pos[kMaxK];
-  float w[kMaxK];
+  const int lane = threadIdx.x;
+  float acc[NV][8];
 #pragma unroll
-  for (int s = 0; s < kMaxK; ++s) {
-    if (s < K) {
-      pos[s] = inverse[(size_t)t * K + s];
-      w[s] = bf16_bits_to_f32(weights[(size_t)t * K + s]);
+  for (int j = 0; j < NV; ++j)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[j][i] = 0.0f;
+
+  auto add_row = [&](const uint4* r, float w) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      float f[8];
+      unpack8(r[j], f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float p = round_bf16_hw(f[i] * w);
+        acc[j][i] = acc[j][i] + p;
+      }
     }
-  }
-  for (int v = threadIdx.x; v < row_vecs; v += blockDim.x) {
-    float acc[8];
+  };
+
+  if (KT > 0) {
+    int pos[KT > 0 ? KT : 1];
+    float w[KT > 0 ? KT : 1];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int s = 0; s < KT; ++s) {
+      pos[s] = inverse[(size_t)t * KT + s];
+      w[s] = bf16_bits_to_f32(weights[(size_t)t * KT + s]);
+    }
+    uint4 rows[KT > 0 ? KT : 1][NV];
 #pragma unroll
-    for (int s = 0; s < kMaxK; ++s) {
-      if (s < K && pos[s] >= 0 && pos[s] < A) {
-        float f[8];
-        unpack8(packed_y[(size_t)pos[s] * row_vecs + v], f);
+    for (int s = 0; s < KT; ++s) {
+      const bool ok = pos[s] >= 0 && pos[s] < A;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float p = round_to_bf16(f[i] * w[s]);
-          acc[i] = acc[i] + p;
-        }
+      for (int j = 0; j < NV; ++j) {
+        const int v = lane + j * 64;
+        rows[s][j] = (ok && v < row_vecs) ? packed_y[(size_t)pos[s] * row_vecs + v] : make_uint4(0, 0, 0, 0);
       }
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = round_to_bf16(acc[i]);
+    for (int s = 0; s < KT; ++s) add_row(rows[s], w[s]);  // a dropped assignment contributes +0
+  } else {
+    for (int s = 0; s < K; ++s) {
+      const int pos = inverse[(size_t)t * K + s];
+      if (pos < 0 || pos >= A) continue;
+      const float w = bf16_bits_to_f32(weights[(size_t)t * K + s]);
+      uint4 r[NV];
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int v = lane + j * 64;
+        r[j] = v < row_vecs ? packed_y[(size_t)pos * row_vecs + v] : make_uint4(0, 0, 0, 0);
+      }
+      add_row(r, w);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = lane + j * 64;
+    if (v >= row_vecs) continue;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[j][i] = round_bf16_hw(acc[j][i]);
     if (shared_y) {
       float f[8];
       unpack8(shared_y[(size_t)t * row_vecs + v], f);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = acc[i] + f[i];  // rounded by pack8
+      for (int i = 0; i < 8; ++i) acc[j][i] = acc[j][i] + f[i];  // rounded by the packing
     }
-    y[(size_t)t * row_vecs + v] = pack8(acc);
+    y[(size_t)t * row_vecs + v] = pack8_hw(acc[j]);
   }
 }
 
@@ -119,18 +164,37 @@ extern "C" int jtmoe_combine(const void* packed_y, const int32_t* inverse, const
   JT_REQUIRE(packed_y && inverse && weights && y, "combine: null pointer argument");
   hipStream_t s = as_stream(stream);
   const int A = (int)(T * K);
-  const bool vec = dtype == JTMOE_BF16 && H % 8 == 0 && aligned16(packed_y) && aligned16(y) &&
+  const bool vec = dtype == JTMOE_BF16 && H % 8 == 0 && H <= 4096 && aligned16(packed_y) && aligned16(y) &&
                    (shared_y == nullptr || aligned16(shared_y));
   if (vec) {
     const int row_vecs = (int)(H / 8);
-    int bx = 64;
-    while (bx < 256 && bx * 2 <= row_vecs) bx *= 2;
-    dim3 block(bx, 256 / bx);
+    dim3 block(64, 4);
     const int grid = (int)((T + block.y - 1) / block.y);
-    combine_bf16_vec_kernel<<<grid, block, 0, s>>>(static_cast<const uint4*>(packed_y), inverse,
-                                                   static_cast<const uint16_t*>(weights),
-                                                   static_cast<const uint4*>(shared_y), (int)T, (int)K, A, row_vecs,
-                                                   static_cast<uint4*>(y));
+    const int nv = (row_vecs + 63) / 64;
+#define JT_COMBINE(NV, KT)                                                                                  \
+  combine_bf16_vec_kernel<NV, KT><<<grid, block, 0, s>>>(                                                   \
+      static_cast<const uint4*>(packed_y), inverse, static_cast<const uint16_t*>(weights),                   \
+      static_cast<const uint4*>(shared_y), (int)T, (int)K, A, row_vecs, static_cast<uint4*>(y))
+#define JT_COMBINE_K(NV)      \
+  if (K == 8)                 \
+    JT_COMBINE(NV, 8);        \
+  else if (K == 2)            \
+    JT_COMBINE(NV, 2);        \
+  else                        \
+    JT_COMBINE(NV, 0)
+    if (nv <= 1) {
+      JT_COMBINE_K(1);
+    } else if (nv <= 2) {
+      JT_COMBINE_K(2);
+    } else if (nv <= 4) {
+      JT_COMBINE_K(4);
+    } else if (nv <= 8) {
+      JT_COMBINE(8, 0);
+    } else {
+      return fail(JTMOE_EUNSUPPORTED, "combine: H=%lld exceeds 4096 on the vector path", (long long)H);
+    }
+#undef JT_COMBINE_K
+#undef JT_COMBINE
   } else {
     dim3 block(64, 4);
     const int grid = (int)((T + block.y - 1) / block.y);

@@ -73,7 +73,7 @@ struct DmaGemmCfg {
   // scheduling options: 16 = request the fragments of MFMA step kk+1 before issuing step kk,
   // 32 = raise the wave priority around the MFMA burst, 64 = ask the scheduler to interleave
   // one MFMA with up to three LDS reads
-  static constexpr int DBG = OPT_;
+  static constexpr int OPT = OPT_;
   static constexpr bool kDual = kDual_;
   static constexpr int BNE = kDual ? 2 * BN : BN;  // columns of the B tile in LDS
   static constexpr int NSUB = BNE / 128;           // 128-column sub-tiles of B
@@ -248,21 +248,21 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     __syncthreads();
     if (kt + NSTAGE - 1 < nk) issue(kt + NSTAGE - 1);
     const unsigned char* st = smem_raw + (kt % NSTAGE) * Cfg::STAGE_BYTES;
-    if (Cfg::DBG & 16) {
+    if (Cfg::OPT & 16) {
       // fragments of step kk+1 are requested before the MFMAs of step kk are issued
       bf16x8_t af[2][TM], bf[2][TN];
       load_frags(st, 0, af[0], bf[0]);
 #pragma unroll
       for (int kk = 0; kk < BK / 16; ++kk) {
         if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-        if (Cfg::DBG & 32) __builtin_amdgcn_s_setprio(1);
+        if (Cfg::OPT & 32) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
           for (int jj = 0; jj < TN; ++jj)
             acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
-        if (Cfg::DBG & 32) __builtin_amdgcn_s_setprio(0);
-        if (Cfg::DBG & 64) {
+        if (Cfg::OPT & 32) __builtin_amdgcn_s_setprio(0);
+        if (Cfg::OPT & 64) {
           // interleave: one MFMA, then up to three LDS reads, repeated
 #pragma unroll
           for (int g = 0; g < TM * TN; ++g) {

@@ -15,8 +15,8 @@
 namespace jtmoe {
 namespace {
 
-constexpr int kRouterTokens = 64;    // tokens per workgroup
-constexpr int kRouterThreads = 256;  // 4 lanes per token in the selection phase
+// A workgroup of NW waves routes 16*NW tokens with 64*NW threads (4 lanes per token in the
+// selection phase).
 constexpr float kFixedScale = 4294967296.0f;  // importance is summed in 32.32 fixed point
 
 // ---- fully specified fp32 sigmoid ------------------------------------------
@@ -91,7 +91,7 @@ struct RouterSmem {
   unsigned long long* imp;  // [E]
 };
 
-__host__ __device__ inline size_t router_smem_bytes(int E, int K) {
+__host__ __device__ inline size_t router_smem_bytes(int E, int K, int kRouterTokens) {
   size_t n = 0;
   n += (size_t)E * 8;                        // imp (first: 8-byte aligned)
   n += (size_t)kRouterTokens * (E + 1) * 4;  // tile
@@ -101,7 +101,7 @@ __host__ __device__ inline size_t router_smem_bytes(int E, int K) {
   return n;
 }
 
-__device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, int K) {
+__device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, int K, int kRouterTokens) {
   RouterSmem s;
   s.imp = reinterpret_cast<unsigned long long*>(base);
   s.tile = reinterpret_cast<float*>(s.imp + E);
@@ -114,12 +114,13 @@ __device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, in
 
 // Everything after the logits tile is in LDS.  `T` is the output element type of
 // the weights.
-template <typename T>
+template <typename T, int NW>
 __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ bias_g, int t0, int tokens,
                                 int E, int K, float route_scale, int32_t* __restrict__ ids_out,
                                 T* __restrict__ weights_out, float* __restrict__ scores_out,
                                 float* __restrict__ logits_out, RouterScratch g) {
 #pragma clang fp contract(off)
+  constexpr int kRouterTokens = 16 * NW, kRouterThreads = 64 * NW;
   const int tid = threadIdx.x;
   const int stride = E + 1;
   const int nrows = min(kRouterTokens, tokens - t0);
@@ -210,13 +211,14 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
 
 // Generic projection: any H, E; fp32 accumulation in k order.
 template <typename T, bool kFromLogits>
-__global__ __launch_bounds__(kRouterThreads) void router_kernel(
+__global__ __launch_bounds__(256) void router_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ logits_in,
     const float* __restrict__ bias, int tokens, int H, int E, int K, float route_scale,
     int32_t* __restrict__ ids, T* __restrict__ weights, float* __restrict__ scores,
     float* __restrict__ logits_out, void* ws) {
+  constexpr int kRouterTokens = 64, kRouterThreads = 256;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  RouterSmem sm = router_smem(smem_raw, E, K);
+  RouterSmem sm = router_smem(smem_raw, E, K, kRouterTokens);
   const int t0 = blockIdx.x * kRouterTokens;
   const int nrows = min(kRouterTokens, tokens - t0);
   const int stride = E + 1;
@@ -234,8 +236,8 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
     sm.tile[t * stride + e] = z;
   }
   __syncthreads();
-  router_epilogue<T>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
-                     router_scratch(ws, E));
+  router_epilogue<T, 4>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
+                        router_scratch(ws, E));
 }
 
 // ---------------------------------------------------------------------------
@@ -256,17 +258,18 @@ constexpr int kBufferFlags = 0x00020000;
 constexpr int kRouterKC = 64;  // k rows of the router matrix per LDS stage
 
 __host__ __device__ inline int router_w_stride(int E) { return E + 32; }  // elements; +64 B between k rows
-__host__ __device__ inline size_t router_mfma_smem_bytes(int E, int K) {
+__host__ __device__ inline size_t router_mfma_smem_bytes(int E, int K, int tokens_per_wg) {
   const size_t w = (size_t)2 * kRouterKC * router_w_stride(E) * 2;
-  const size_t ep = router_smem_bytes(E, K);
+  const size_t ep = router_smem_bytes(E, K, tokens_per_wg);
   return w > ep ? w : ep;
 }
 
-template <int NB>
-__global__ __launch_bounds__(kRouterThreads) void router_mfma_kernel(
+template <int NB, int NW>
+__global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
     int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
     float* __restrict__ scores, float* __restrict__ logits_out, void* ws) {
+  constexpr int kRouterTokens = 16 * NW, kRouterThreads = 64 * NW;
   constexpr int E = NB * 16;
   constexpr int WS = E + 32;                      // LDS row stride of the staged matrix (elements)
   constexpr int W_CHUNKS = kRouterKC * E / 8;     // 16-byte chunks per stage
@@ -354,7 +357,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_mfma_kernel(
 
   // logits (rounded to bf16, as the projection's output dtype) -> LDS tile; value i of lane l
   // is token row 4*(l/16) + i, expert nb*16 + l%16
-  RouterSmem sm = router_smem(smem_raw, E, K);
+  RouterSmem sm = router_smem(smem_raw, E, K, kRouterTokens);
   const int stride = E + 1;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
@@ -362,8 +365,8 @@ __global__ __launch_bounds__(kRouterThreads) void router_mfma_kernel(
     for (int i = 0; i < 4; ++i)
       sm.tile[(wave * 16 + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = round_to_bf16(acc[nb][i]);
   __syncthreads();
-  router_epilogue<bf16_raw>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
-                            router_scratch(ws, E));
+  router_epilogue<bf16_raw, NW>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
+                                router_scratch(ws, E));
 }
 
 template <typename KernelT>
@@ -380,24 +383,34 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
                   int64_t H, int64_t E, int64_t K, double route_scale, int32_t* ids, void* weights,
                   float* scores, float* counts, float* importance, float* logits_out, void* ws,
                   hipStream_t stream) {
-  const int blocks = (int)((tokens + kRouterTokens - 1) / kRouterTokens);
   const bool mfma = Elem<T>::is_bf16 && !kFromLogits && H % kRouterKC == 0 && H * E < ((int64_t)1 << 30) &&
                     (E == 16 || E == 32 || E == 64 || E == 128 || E == 256) && aligned16(x) && aligned16(w);
   if (mfma) {
-    const size_t smem = router_mfma_smem_bytes((int)E, (int)K);
+    // two waves (32 tokens) per workgroup: several workgroups share a CU and hide each other's
+    // projection / selection phases; one wave when there are too few tokens to fill the chip
+    const int nw = tokens >= 8192 ? 2 : 1;
+    const int tok = 16 * nw;
+    const int blocks = (int)((tokens + tok - 1) / tok);
+    const size_t smem = router_mfma_smem_bytes((int)E, (int)K, tok);
     if (smem > 160 * 1024) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
     router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
     if (tokens > 0) {
-#define JT_ROUTER_CASE(NB)                                                                                   \
-  case NB * 16: {                                                                                            \
-    auto kernel = router_mfma_kernel<NB>;                                                                    \
+#define JT_ROUTER_LAUNCH(NB, NW)                                                                             \
+  {                                                                                                          \
+    auto kernel = router_mfma_kernel<NB, NW>;                                                                \
     int rc = set_max_smem(kernel, smem);                                                                     \
     if (rc) return rc;                                                                                       \
-    kernel<<<blocks, kRouterThreads, smem, stream>>>(                                                        \
+    kernel<<<blocks, 64 * NW, smem, stream>>>(                                                               \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
         (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws);                   \
-    break;                                                                                                   \
   }
+#define JT_ROUTER_CASE(NB)        \
+  case NB * 16:                   \
+    if (nw == 2)                  \
+      JT_ROUTER_LAUNCH(NB, 2)     \
+    else                          \
+      JT_ROUTER_LAUNCH(NB, 1)     \
+    break;
       switch ((int)E) {
         JT_ROUTER_CASE(1)
         JT_ROUTER_CASE(2)
@@ -406,16 +419,18 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
         JT_ROUTER_CASE(16)
       }
 #undef JT_ROUTER_CASE
+#undef JT_ROUTER_LAUNCH
     }
   } else {
-    const size_t smem = router_smem_bytes((int)E, (int)K);
+    const int blocks = (int)((tokens + 63) / 64);
+    const size_t smem = router_smem_bytes((int)E, (int)K, 64);
     if (smem > 160 * 1024) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
     auto kernel = router_kernel<T, kFromLogits>;
     int rc = set_max_smem(kernel, smem);
     if (rc) return rc;
     router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
     if (tokens > 0)
-      kernel<<<blocks, kRouterThreads, smem, stream>>>(
+      kernel<<<blocks, 256, smem, stream>>>(
           static_cast<const T*>(x), static_cast<const T*>(w), logits_in, bias, (int)tokens, (int)H, (int)E, (int)K,
           (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws);
   }
