@@ -23,10 +23,11 @@ from research_amd.errors import ContractError
 CACHE_SCHEMA_VERSION = 1
 MANIFEST_NAME = "manifest.json"
 LIBRARY_NAME = "libjtmoe.so"
+NATIVE_TEST_NAME = "gemm_check"
 ARCH = "gfx950"
 SOURCE_FILES = (
     "api.hip", "router.hip", "dispatch.hip", "combine.hip", "grouped_gemm.hip",
-    "common.hpp", "gemm_common.hpp", "grouped_gemm_dma.hpp",
+    "common.hpp", "gemm_common.hpp", "grouped_gemm_dma.hpp", "native/gemm_check.hip",
 )
 
 
@@ -107,7 +108,14 @@ def compile_kernels(root: str | Path | None = None, *, jobs: int = 8, clean: boo
                     "arch": ARCH,
                     "compiler": _compiler_version(hipcc),
                     "sources": {name: _sha256(source_dir() / name) for name in SOURCE_FILES},
-                }
+                },
+                "standalone_test": {
+                    "path": NATIVE_TEST_NAME,
+                    "sha256": _sha256(out_dir / NATIVE_TEST_NAME),
+                    "bytes": (out_dir / NATIVE_TEST_NAME).stat().st_size,
+                    "kind": "standalone_test",
+                    "arch": ARCH,
+                },
             }
         },
     }

@@ -169,10 +169,6 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   return JTMOE_OK;
 }
 
-// 256 x 256 output tiles (gate and up share the A tile: 128 + 128 columns), 64-deep k steps,
-// two LDS stages, 8 waves
-using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16>;
-using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64>;
 
 inline bool fast_ok(const void* a, const void* b0, const void* b1, const void* c, int64_t Kdim, int64_t N) {
   return Kdim % 64 == 0 && N % 8 == 0 && Kdim * N < ((int64_t)1 << 30) && aligned16(a) && aligned16(b0) && (b1 == nullptr || aligned16(b1)) &&

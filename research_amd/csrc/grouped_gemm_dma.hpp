@@ -327,4 +327,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   }
 }
 
+// The two configurations the library launches: 256 x 256 output tiles (gate and up share the A
+// tile: 128 + 128 columns), 64-deep k steps, two LDS stages, 8 waves.
+using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16>;
+using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64>;
+
 }  // namespace jtmoe
