@@ -60,3 +60,17 @@ def test_dtype_names():
     assert moe.dtype_from_name("bfloat16") is torch.bfloat16
     with pytest.raises(ContractError):
         moe.dtype_from_name("float16")
+
+
+def test_jax_ffi_stub_fails_loudly_without_jax():
+    import importlib.util
+
+    from research_amd import jax_ffi
+
+    if importlib.util.find_spec("jax") is not None:
+        pytest.skip("jax is installed here")
+    with pytest.raises(ContractError, match="jax is not installed"):
+        jax_ffi.register_moe()
+    assert set(jax_ffi.TARGETS.values()) == {
+        "JaxtitanMoeForward", "JaxtitanMoeRouter", "JaxtitanMoeDispatch", "JaxtitanMoeGroupedSwiglu",
+        "JaxtitanMoeCombine"}
