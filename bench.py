@@ -218,17 +218,37 @@ def main() -> int:
         return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
 
     gate_up_tf = tflops(work["gate_up_flops"], stage_ms["gate_up"])
-    roofline = dict(
-        kernel="grouped gate/up GEMM + SwiGLU (routed experts)",
-        bound="mfma",
-        achieved=gate_up_tf,
-        peak=peak,
-        unit="TFLOP/s",
-        frac=gate_up_tf / peak,
-        traffic=measured_traffic(args.config, "gate_up"),
-        avg_launch_ms=stage_ms["gate_up"],
-        flops_per_launch=work["gate_up_flops"],
-    )
+    active = sum(1 for g in group_sizes if g > 0)
+    elem = 2 if cfg["dtype"] == "bf16" else 4
+    # bytes the gate/up launch must move: the gate and up matrices of every expert that received
+    # a row, each token row once, the activation rows written
+    gate_up_bytes = (2 * active * cfg["H"] * cfg["I"] + T * cfg["H"] + A_rows * cfg["I"]) * elem
+    if args.config == "C5":
+        # a few rows per expert: the launch streams the expert matrices once and is bound by HBM
+        gate_up_gbs = gbs(gate_up_bytes, stage_ms["gate_up"])
+        roofline = dict(
+            kernel="grouped gate/up GEMM + SwiGLU (routed experts, weight streaming)",
+            bound="hbm",
+            achieved=gate_up_gbs,
+            peak=HBM_PEAK_GBS,
+            unit="GB/s",
+            frac=gate_up_gbs / HBM_PEAK_GBS,
+            traffic=measured_traffic(args.config, "gate_up"),
+            avg_launch_ms=stage_ms["gate_up"],
+            bytes_per_launch=gate_up_bytes,
+        )
+    else:
+        roofline = dict(
+            kernel="grouped gate/up GEMM + SwiGLU (routed experts)",
+            bound="mfma",
+            achieved=gate_up_tf,
+            peak=peak,
+            unit="TFLOP/s",
+            frac=gate_up_tf / peak,
+            traffic=measured_traffic(args.config, "gate_up"),
+            avg_launch_ms=stage_ms["gate_up"],
+            flops_per_launch=work["gate_up_flops"],
+        )
     stages = dict(
         ms=stage_ms,
         standalone_dispatch_ms=dispatch_ms,

@@ -170,6 +170,10 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
 }
 
 
+// Mean rows per group below which the 64-row tiles are used.
+constexpr int64_t kSmallGroupRows = 128;
+inline bool small_groups(int64_t rows, int64_t E) { return rows < kSmallGroupRows * E; }
+
 inline bool fast_ok(const void* a, const void* b0, const void* b1, const void* c, int64_t Kdim, int64_t N) {
   return Kdim % 64 == 0 && N % 8 == 0 && Kdim * N < ((int64_t)1 << 30) && aligned16(a) && aligned16(b0) && (b1 == nullptr || aligned16(b1)) &&
          aligned16(c);
@@ -182,9 +186,12 @@ int launch_pair(const void* x, const void* gate, const void* up, const void* dow
                 int64_t x_rows = 0) {
   if (rows == 0) return JTMOE_OK;
   int rc;
+  const bool small = small_groups(rows, E);
   if (Elem<T>::is_bf16 && fast_ok(x, gate, up, act, H, I))
-    rc = launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map, row_div,
-                                x_rows);
+    rc = small ? launch_fast<GateUpSmallCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
+                                             row_div, x_rows)
+               : launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
+                                        row_div, x_rows);
   else if (row_map != nullptr)
     return fail(JTMOE_EUNSUPPORTED, "grouped_swiglu_gather: shape or alignment outside the gather-on-load path");
   else
@@ -192,7 +199,8 @@ int launch_pair(const void* x, const void* gate, const void* up, const void* dow
   if (rc) return rc;
   stage_mark(first_stage, stream);
   if (Elem<T>::is_bf16 && fast_ok(act, down, nullptr, y, I, H))
-    rc = launch_fast<DownCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
+    rc = small ? launch_fast<DownSmallCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream)
+               : launch_fast<DownCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
   else
     rc = launch_generic<T, false>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
   if (rc) return rc;

@@ -331,5 +331,10 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
 // tile: 128 + 128 columns), 64-deep k steps, two LDS stages, 8 waves.
 using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16>;
 using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64>;
+// Few rows per group (decode-sized batches): the layer streams every expert matrix once and
+// is bound by HBM, so the tiles are only 64 rows tall to keep the padded-row MFMA work below
+// the time the weights take to arrive.  Two workgroups fit the LDS of one CU.
+using GateUpSmallCfg = DmaGemmCfg<64, 128, 64, 2, 4, true, 2, 16>;
+using DownSmallCfg = DmaGemmCfg<64, 256, 64, 2, 4, false, 2, 16>;
 
 }  // namespace jtmoe

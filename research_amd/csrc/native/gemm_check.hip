@@ -196,6 +196,17 @@ int main(int argc, char** argv) {
     ok &= check<DownCfg>("down dense", p, true);
     release(p);
   }
+  {
+    Problem p = make(16, 150, 512, 392, 6, true, 0, 1.0f);  // a handful of rows per group: the 64-row tiles
+    ok &= check<GateUpSmallCfg>("gate/up few rows per group", p);
+    ok &= check<DownSmallCfg>("down few rows per group", p);
+    release(p);
+  }
+  {
+    Problem p = make(5, 300, 512, 384, 7, true, 3, 1.0f);
+    ok &= check<GateUpSmallCfg>("gate/up few rows, gather on load", p);
+    release(p);
+  }
   if (ok && argc > 1 && !strcmp(argv[1], "time")) {
     for (float scale : {1.0f, 0.0f}) {
       printf("-- operand data: %s\n", scale > 0 ? "N(0,1) activations, N(0,0.05) weights" : "all zeros");
@@ -206,6 +217,15 @@ int main(int argc, char** argv) {
       timeit<DownCfg>("down 64 groups", d, 20);
       release(d);
     }
+    // decode-sized batch: 8 rows per group, bound by streaming the expert matrices
+    Problem g = make(64, 512, 2048, 1408, 8, false, 0, 1.0f);
+    timeit<GateUpCfg>("gate/up 64 groups, 256-row tiles", g, 20);
+    timeit<GateUpSmallCfg>("gate/up 64 groups, 64-row tiles", g, 20);
+    release(g);
+    Problem d = make(64, 512, 1408, 2048, 9, false, 0, 1.0f);
+    timeit<DownCfg>("down 64 groups, 256-row tiles", d, 20);
+    timeit<DownSmallCfg>("down 64 groups, 64-row tiles", d, 20);
+    release(d);
   }
   printf(ok ? "PASS\n" : "FAIL\n");
   return ok ? 0 : 1;

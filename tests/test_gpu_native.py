@@ -20,4 +20,4 @@ def test_native_gemm_check_passes(gpu):
     print(proc.stdout, flush=True)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert proc.stdout.strip().endswith("PASS")
-    assert proc.stdout.count("bad=0") == 5
+    assert proc.stdout.count("bad=0") == proc.stdout.count("case ") >= 8
