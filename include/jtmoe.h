@@ -221,6 +221,114 @@ int jtmoe_moe_forward_timed(const void* x, const void* w_router, const float* ex
                             void* workspace, size_t workspace_bytes, void* stream,
                             float* stage_ms);
 
+/* ------------------------------------------------------------------------------------------
+ * Training: forward passes that keep residuals, and the vector-Jacobian products.
+ *
+ * The reference trains SparseMoE through JAX automatic differentiation and requires a
+ * forward-only kernel to bring its own VJP before it may replace a training component
+ * (docs/kernel_backend_design.md:120-128).  These entry points are that VJP, operator by
+ * operator; the gradient tests of the reference's expert dispatcher are the specification
+ * (tests/jaxtitan/test_model.py:549-691: gradients with respect to x, route weights, gate,
+ * up and down; repeated calls must return identical bits).
+ *
+ * Residuals: gate_pre = round(Xp Wg[e]) and up_pre = round(Xp Wu[e]), both [A, I] in the
+ * compute dtype (packed row order), and the same two for the shared experts, [T, Is].
+ * Gradients of rounding steps are passed straight through.  Gradient outputs have the
+ * compute dtype and the shape of what they differentiate.
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * jtmoe_grouped_swiglu / jtmoe_grouped_swiglu_gather that also store gate_pre and up_pre.
+ * source_order != NULL: x is [T, H] token-major and packed row j reads token
+ * source_order[j] / K (A = T*K); source_order == NULL: x is already packed, A = T rows.
+ */
+int jtmoe_grouped_swiglu_train(const void* x, const int32_t* source_order,
+                               const void* gate, const void* up, const void* down,
+                               const int32_t* group_sizes, const int32_t* offsets,
+                               int64_t T, int64_t K, int64_t H, int64_t I, int64_t E, int dtype,
+                               void* gate_pre, void* up_pre, void* act, void* packed_y, void* stream);
+
+/* jtmoe_shared_swiglu that also stores gate_pre and up_pre ([T, Is]). */
+int jtmoe_shared_swiglu_train(const void* x, const void* gate, const void* up, const void* down,
+                              int64_t T, int64_t H, int64_t Is, int dtype,
+                              void* gate_pre, void* up_pre, void* act, void* shared_y, void* stream);
+
+/*
+ * VJP of dispatch -> grouped SwiGLU -> combine (moe.py:583-671) for the cotangent dy [T, H]:
+ *   dx [T, H]        = sum_s dXp[inverse[t,s]]  (+ dx_extra, if given: e.g. the shared experts'
+ *                      and the router's contribution to the gradient of x)
+ *   d_weights [T, K] = <dy[t], Yp[inverse[t,s]]>
+ *   d_gate, d_up [E, H, I], d_down [E, I, H]; experts without rows get zeros.
+ * weights are the route weights [T, K] of the forward pass.
+ */
+size_t jtmoe_experts_backward_workspace_bytes(int64_t T, int64_t K, int64_t H, int64_t I, int dtype);
+int jtmoe_experts_backward(const void* x, const void* dy,
+                           const int32_t* source_order, const int32_t* inverse, const void* weights,
+                           const int32_t* group_sizes, const int32_t* offsets,
+                           const void* gate, const void* up, const void* down,
+                           const void* gate_pre, const void* up_pre,
+                           int64_t T, int64_t K, int64_t H, int64_t I, int64_t E, int dtype,
+                           const void* dx_extra,
+                           void* dx, void* d_weights, void* d_gate, void* d_up, void* d_down,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* VJP of SharedSwiGLU.__call__ (moe.py:361-364): dx [T, H], d_gate, d_up [H, Is], d_down [Is, H]. */
+size_t jtmoe_shared_backward_workspace_bytes(int64_t T, int64_t Is, int dtype);
+int jtmoe_shared_backward(const void* x, const void* dy,
+                          const void* gate, const void* up, const void* down,
+                          const void* gate_pre, const void* up_pre,
+                          int64_t T, int64_t H, int64_t Is, int dtype,
+                          void* dx, void* d_gate, void* d_up, void* d_down,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * VJP of SigmoidTopKRouter.__call__ (moe.py:131-147) for the cotangents d_weights [T, K]
+ * (compute dtype) and, optionally, d_scores [T, E] (fp32; NULL = zeros), e.g. from an
+ * auxiliary loss on the scores.  scores and expert_ids are the forward's outputs.  The
+ * selection itself and the expert bias carry no gradient (moe.py:139-140).
+ *   dx [T, H], d_w_router [H, E].
+ */
+size_t jtmoe_router_backward_workspace_bytes(int64_t T, int64_t E, int dtype);
+int jtmoe_router_backward(const void* x, const void* w_router,
+                          const float* scores, const int32_t* expert_ids,
+                          const void* d_weights, const float* d_scores, double route_scale,
+                          int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
+                          void* dx, void* d_w_router,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The layer: jtmoe_moe_forward that also stores the residuals, and the VJP of
+ * SparseMoE.forward_with_output (moe.py:409-430) for the cotangents dy [T, H] and
+ * d_scores [T, E] (NULL = zeros).  Is == 0: pass NULL for every shared-expert argument.
+ */
+int jtmoe_moe_forward_train(const void* x, const void* w_router, const float* expert_bias,
+                            const void* gate, const void* up, const void* down,
+                            const void* shared_gate, const void* shared_up, const void* shared_down,
+                            int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                            double route_scale, int dtype,
+                            void* y, int32_t* expert_ids, void* weights, float* scores,
+                            float* expert_counts, float* importance,
+                            int32_t* group_sizes, int32_t* offsets,
+                            int32_t* source_order, int32_t* inverse,
+                            void* gate_pre, void* up_pre, void* shared_gate_pre, void* shared_up_pre,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+size_t jtmoe_moe_backward_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                                          int dtype);
+int jtmoe_moe_backward(const void* x, const void* dy, const float* d_scores,
+                       const void* w_router, const void* gate, const void* up, const void* down,
+                       const void* shared_gate, const void* shared_up, const void* shared_down,
+                       const float* scores, const int32_t* expert_ids, const void* weights,
+                       const int32_t* source_order, const int32_t* inverse,
+                       const int32_t* group_sizes, const int32_t* offsets,
+                       const void* gate_pre, const void* up_pre,
+                       const void* shared_gate_pre, const void* shared_up_pre,
+                       double route_scale,
+                       int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype,
+                       void* dx, void* d_w_router, void* d_gate, void* d_up, void* d_down,
+                       void* d_shared_gate, void* d_shared_up, void* d_shared_down,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

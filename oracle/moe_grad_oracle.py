@@ -1,0 +1,163 @@
+"""CPU oracle for the backward pass of the MoE expert layer.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker, never the product: only ``tests/`` may import it.
+
+The reference has no hand-written backward: it differentiates
+``SparseMoE.forward_with_output`` (src/jaxtitan/models/components/moe.py:409-430)
+with ``jax.grad`` (jax 0.10.0, pinned in the reference's ``uv.lock``; absent from
+this environment).  What that yields is fixed by the chain rule applied to the
+forward formulas, which this module restates in float64, operator by operator:
+
+* ``experts_backward``  <- VJP of dispatch + ``ExpertSwiGLU`` + combine   moe.py:583-671
+* ``shared_backward``   <- VJP of ``SharedSwiGLU.__call__``               moe.py:361-364
+* ``router_backward``   <- VJP of ``SigmoidTopKRouter.__call__``          moe.py:131-147
+* ``moe_backward``      <- VJP of the layer (sum of the three over x)     moe.py:409-430
+
+Inputs are taken as they are (callers round them to the compute dtype first);
+all arithmetic is float64 and nothing is rounded on the way, i.e. this is the
+exact gradient of the un-rounded forward function at the given inputs.  The
+selection (``expert_ids``) is piecewise constant and carries no gradient, and the
+expert bias only enters the selection (moe.py:139-140).
+
+Parity status (exercised in ``tests/test_oracle_grad.py``):
+
+* experts_backward: pinned by central finite differences of the dense
+  formulation the reference's own gradient test differentiates
+  (tests/jaxtitan/test_model.py:596-603: gather the selected expert matrices,
+  three einsums, weighted sum) on that test's inputs and its four routing
+  patterns (balanced, one expert unused, all on one expert, duplicate routes),
+  for all five differentiable arguments.
+* shared_backward: pinned by finite differences of a plain two-matmul SwiGLU.
+* router_backward: pinned by finite differences of the float64 closed form
+  ``scale * p / (sum p + 1e-20)`` with the selection held fixed, including the
+  extra cotangent on the scores.
+* moe_backward: pinned by finite differences of the float64 layer built from the
+  three closed forms above with the selection held fixed.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+
+
+def _f64(a):
+    return np.asarray(a, dtype=np.float64)
+
+
+def _sigmoid(z):
+    return 1.0 / (1.0 + np.exp(-z))
+
+
+@dataclass
+class ExpertsGrad:
+    dx: np.ndarray  # [T,H]
+    d_weights: np.ndarray  # [T,K]
+    d_gate: np.ndarray  # [E,H,I]
+    d_up: np.ndarray  # [E,H,I]
+    d_down: np.ndarray  # [E,I,H]
+
+
+def experts_backward(x, expert_ids, weights, gate, up, down, dy) -> ExpertsGrad:
+    """Gradient of y[t] = sum_s w[t,s] * (silu(x[t] Wg[e]) * (x[t] Wu[e])) Wd[e], e = ids[t,s]."""
+    x, weights, gate, up, down, dy = (_f64(a) for a in (x, weights, gate, up, down, dy))
+    ids = np.asarray(expert_ids)
+    E = gate.shape[0]
+    dx = np.zeros_like(x)
+    d_weights = np.zeros_like(weights)
+    d_gate, d_up, d_down = np.zeros_like(gate), np.zeros_like(up), np.zeros_like(down)
+    for e in range(E):
+        t_idx, s_idx = np.nonzero(ids == e)
+        if t_idx.size == 0:
+            continue
+        xe, dye = x[t_idx], dy[t_idx]
+        g, u = xe @ gate[e], xe @ up[e]
+        sig = _sigmoid(g)
+        h = g * sig * u
+        yp = h @ down[e]
+        w = weights[t_idx, s_idx][:, None]
+        d_weights[t_idx, s_idx] = np.sum(dye * yp, axis=-1)
+        dyp = dye * w
+        dh = dyp @ down[e].T
+        d_down[e] = h.T @ dyp
+        dg = dh * u * sig * (1.0 + g * (1.0 - sig))
+        du = dh * g * sig
+        d_gate[e] = xe.T @ dg
+        d_up[e] = xe.T @ du
+        np.add.at(dx, t_idx, dg @ gate[e].T + du @ up[e].T)
+    return ExpertsGrad(dx, d_weights, d_gate, d_up, d_down)
+
+
+@dataclass
+class SharedGrad:
+    dx: np.ndarray
+    d_gate: np.ndarray
+    d_up: np.ndarray
+    d_down: np.ndarray
+
+
+def shared_backward(x, gate, up, down, dy) -> SharedGrad:
+    """Gradient of y = (silu(x Wg) * (x Wu)) Wd."""
+    x, gate, up, down, dy = (_f64(a) for a in (x, gate, up, down, dy))
+    g, u = x @ gate, x @ up
+    sig = _sigmoid(g)
+    h = g * sig * u
+    dh = dy @ down.T
+    dg = dh * u * sig * (1.0 + g * (1.0 - sig))
+    du = dh * g * sig
+    return SharedGrad(dg @ gate.T + du @ up.T, x.T @ dg, x.T @ du, h.T @ dy)
+
+
+@dataclass
+class RouterGrad:
+    dx: np.ndarray  # [T,H]
+    d_w_router: np.ndarray  # [H,E]
+    d_logits: np.ndarray  # [T,E]
+
+
+def router_backward(x, w_router, expert_ids, d_weights, d_scores, route_scale, scores=None) -> RouterGrad:
+    """Gradient of weights = scale * p / (sum p + 1e-20), p = sigmoid(x W)[ids], plus a cotangent on the scores.
+
+    ``scores`` overrides sigmoid(x W) (pass the forward's own scores to follow its rounding).
+    """
+    x, w_router, d_weights = _f64(x), _f64(w_router), _f64(d_weights)
+    ids = np.asarray(expert_ids)
+    T = x.shape[0]
+    sc = _sigmoid(x @ w_router) if scores is None else _f64(scores)
+    rows = np.arange(T)[:, None]
+    p = sc[rows, ids]
+    S = p.sum(-1, keepdims=True) + 1e-20
+    dp = route_scale * (d_weights / S - np.sum(d_weights * p, axis=-1, keepdims=True) / S**2)
+    d_sc = np.zeros_like(sc) if d_scores is None else _f64(d_scores).copy()
+    np.add.at(d_sc, (np.broadcast_to(rows, ids.shape), ids), dp)
+    d_logits = d_sc * sc * (1.0 - sc)
+    return RouterGrad(d_logits @ w_router.T, x.T @ d_logits, d_logits)
+
+
+@dataclass
+class LayerGrad:
+    dx: np.ndarray
+    d_w_router: np.ndarray
+    d_gate: np.ndarray
+    d_up: np.ndarray
+    d_down: np.ndarray
+    d_shared: tuple | None  # (d_gate, d_up, d_down) of the shared experts
+    d_weights: np.ndarray  # [T,K], the intermediate cotangent of the route weights
+
+
+def moe_backward(x, w_router, gate, up, down, shared, expert_ids, weights, dy, d_scores, route_scale,
+                 scores=None) -> LayerGrad:
+    """Gradient of the layer y = routed(x) + shared(x) for the cotangents dy and d_scores.
+
+    ``weights`` are the route weights the forward used; ``expert_ids`` its selection.
+    """
+    eg = experts_backward(x, expert_ids, weights, gate, up, down, dy)
+    rg = router_backward(x, w_router, expert_ids, eg.d_weights, d_scores, route_scale, scores)
+    dx = eg.dx + rg.dx
+    d_shared = None
+    if shared is not None:
+        sg = shared_backward(x, shared[0], shared[1], shared[2], dy)
+        dx = dx + sg.dx
+        d_shared = (sg.d_gate, sg.d_up, sg.d_down)
+    return LayerGrad(dx, rg.d_w_router, eg.d_gate, eg.d_up, eg.d_down, d_shared, eg.d_weights)

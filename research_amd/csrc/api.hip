@@ -245,14 +245,18 @@ extern "C" size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t
   return carve_layer(nullptr, T, H, E, K, I, Is, dtype).total;
 }
 
-extern "C" int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_bias, const void* gate,
-                                 const void* up, const void* down, const void* shared_gate, const void* shared_up,
-                                 const void* shared_down, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I,
-                                 int64_t Is, double route_scale, int dtype, void* y, int32_t* expert_ids,
-                                 void* weights, float* scores, float* expert_counts, float* importance,
-                                 int32_t* group_sizes, int32_t* offsets, int32_t* source_order, int32_t* inverse,
-                                 void* workspace, size_t workspace_bytes, void* stream) {
+// gate_pre .. shared_up_pre: where the training forward keeps the four rounded products that the
+// backward pass reads; all null for the plain forward
+static int moe_forward_impl(const void* x, const void* w_router, const float* expert_bias, const void* gate,
+                            const void* up, const void* down, const void* shared_gate, const void* shared_up,
+                            const void* shared_down, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I,
+                            int64_t Is, double route_scale, int dtype, void* y, int32_t* expert_ids, void* weights,
+                            float* scores, float* expert_counts, float* importance, int32_t* group_sizes,
+                            int32_t* offsets, int32_t* source_order, int32_t* inverse, void* workspace,
+                            size_t workspace_bytes, void* stream, void* gate_pre, void* up_pre,
+                            void* shared_gate_pre, void* shared_up_pre) {
   clear_error();
+  const bool train = gate_pre != nullptr;
   JT_REQUIRE(dtype_ok(dtype), "moe_forward: unknown dtype %d", dtype);
   JT_REQUIRE(T >= 0 && H > 0 && E > 0 && K > 0 && I > 0 && Is >= 0, "moe_forward: shape out of range");
   JT_REQUIRE((Is == 0) == (shared_gate == nullptr) && (Is == 0) == (shared_up == nullptr) &&
@@ -269,13 +273,16 @@ extern "C" int jtmoe_moe_forward(const void* x, const void* w_router, const floa
   stage_mark(kStageRouter, as_stream(stream));
   // where the GEMM can apply the permutation while it fetches its A tiles, the permuted copy of
   // x is never written: dispatch then only computes the histogram, offsets and permutation
-  const bool gather = T > 0 && jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) &&
+  const bool gather = train || (T > 0 && jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) &&
                       (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(gate) & 15u) == 0 &&
-                      (reinterpret_cast<uintptr_t>(up) & 15u) == 0 && (reinterpret_cast<uintptr_t>(down) & 15u) == 0;
+                      (reinterpret_cast<uintptr_t>(up) & 15u) == 0 && (reinterpret_cast<uintptr_t>(down) & 15u) == 0);
   rc = jtmoe_dispatch(expert_ids, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes, offsets,
                       source_order, inverse, w.packed_x, w.dispatch, w.dispatch_bytes, stream);
   if (rc) return rc;
-  if (gather)
+  if (train)
+    rc = jtmoe_grouped_swiglu_train(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
+                                    gate_pre, up_pre, w.act, w.packed_y, stream);
+  else if (gather)
     rc = jtmoe_grouped_swiglu_gather(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
                                      w.act, w.packed_y, stream);
   else
@@ -283,13 +290,51 @@ extern "C" int jtmoe_moe_forward(const void* x, const void* w_router, const floa
                               w.packed_y, stream);
   if (rc) return rc;
   if (Is > 0) {
-    rc = jtmoe_shared_swiglu(x, shared_gate, shared_up, shared_down, T, H, Is, dtype, w.shared_act, w.shared_y,
-                             stream);
+    if (train)
+      rc = jtmoe_shared_swiglu_train(x, shared_gate, shared_up, shared_down, T, H, Is, dtype, shared_gate_pre,
+                                     shared_up_pre, w.shared_act, w.shared_y, stream);
+    else
+      rc = jtmoe_shared_swiglu(x, shared_gate, shared_up, shared_down, T, H, Is, dtype, w.shared_act, w.shared_y,
+                               stream);
     if (rc) return rc;
   }
   rc = jtmoe_combine(w.packed_y, inverse, weights, Is > 0 ? w.shared_y : nullptr, T, H, K, dtype, y, stream);
   stage_mark(kStageCombine, as_stream(stream));
   return rc;
+}
+
+extern "C" int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_bias, const void* gate,
+                                 const void* up, const void* down, const void* shared_gate, const void* shared_up,
+                                 const void* shared_down, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I,
+                                 int64_t Is, double route_scale, int dtype, void* y, int32_t* expert_ids,
+                                 void* weights, float* scores, float* expert_counts, float* importance,
+                                 int32_t* group_sizes, int32_t* offsets, int32_t* source_order, int32_t* inverse,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  return moe_forward_impl(x, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H, E, K, I,
+                          Is, route_scale, dtype, y, expert_ids, weights, scores, expert_counts, importance,
+                          group_sizes, offsets, source_order, inverse, workspace, workspace_bytes, stream, nullptr,
+                          nullptr, nullptr, nullptr);
+}
+
+extern "C" int jtmoe_moe_forward_train(const void* x, const void* w_router, const float* expert_bias,
+                                       const void* gate, const void* up, const void* down, const void* shared_gate,
+                                       const void* shared_up, const void* shared_down, int64_t T, int64_t H,
+                                       int64_t E, int64_t K, int64_t I, int64_t Is, double route_scale, int dtype,
+                                       void* y, int32_t* expert_ids, void* weights, float* scores,
+                                       float* expert_counts, float* importance, int32_t* group_sizes,
+                                       int32_t* offsets, int32_t* source_order, int32_t* inverse, void* gate_pre,
+                                       void* up_pre, void* shared_gate_pre, void* shared_up_pre, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  if (T > 0 && (gate_pre == nullptr || up_pre == nullptr || (Is > 0 && (!shared_gate_pre || !shared_up_pre)))) {
+    clear_error();
+    return fail(JTMOE_EINVAL, "moe_forward_train: null residual buffer");
+  }
+  // the address of a local stands in for the residual pointers when there are no tokens
+  int none = 0;
+  return moe_forward_impl(x, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H, E, K, I,
+                          Is, route_scale, dtype, y, expert_ids, weights, scores, expert_counts, importance,
+                          group_sizes, offsets, source_order, inverse, workspace, workspace_bytes, stream,
+                          gate_pre ? gate_pre : &none, up_pre ? up_pre : &none, shared_gate_pre, shared_up_pre);
 }
 
 extern "C" int jtmoe_moe_forward_timed(const void* x, const void* w_router, const float* expert_bias,

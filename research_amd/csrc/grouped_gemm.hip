@@ -55,8 +55,10 @@ template <typename T, bool kDual>
 __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(
     const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
     const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E, int dense_rows, int Kdim,
-    int N, int ntiles_n) {
+    int N, int ntiles_n, const int32_t* __restrict__ row_map, int row_div, T* __restrict__ save0,
+    T* __restrict__ save1) {
   __shared__ __align__(16) T As[GBM][GBK + GPAD];
+  __shared__ int a_row_of[GBM];  // row of A behind tile row r (through the row map, if there is one)
   __shared__ __align__(16) T Bs0[GBN][GBK + GPAD];
   __shared__ __align__(16) T Bs1[kDual ? GBN : 1][GBK + GPAD];
 
@@ -82,13 +84,15 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(
 
   T zero;
   __builtin_memset(&zero, 0, sizeof(T));
+  if (tid < GBM && tid < tr.rows) a_row_of[tid] = row_map ? row_map[tr.row0 + tid] / row_div : tr.row0 + tid;
+  __syncthreads();
 
   for (int k0 = 0; k0 < Kdim; k0 += GBK) {
     for (int idx = tid; idx < GBM * GBK; idx += 256) {
       const int r = idx / GBK, c = idx - r * GBK;
       const int gk = k0 + c;
       T v = zero;
-      if (r < tr.rows && gk < Kdim) v = A[(size_t)(tr.row0 + r) * Kdim + gk];
+      if (r < tr.rows && gk < Kdim) v = A[(size_t)a_row_of[r] * Kdim + gk];
       As[r][c] = v;
     }
     for (int idx = tid; idx < GBK * GBN; idx += 256) {
@@ -117,6 +121,10 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(
           const float g = Elem<T>::round(acc0[i]);
           const float u = Elem<T>::round(acc1[i]);
           v = silu_fast(g) * u;
+          if (save0) {
+            Elem<T>::store(save0 + (size_t)(tr.row0 + r) * N + col, g);
+            Elem<T>::store(save1 + (size_t)(tr.row0 + r) * N + col, u);
+          }
         } else {
           v = acc0[i];
         }
@@ -133,21 +141,24 @@ inline int64_t max_m_tiles(int64_t rows, int64_t groups, int BM) {
 
 template <typename T, bool kDual>
 int launch_generic(const void* a, const void* b0, const void* b1, void* c, const int32_t* group_sizes,
-                   const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream) {
+                   const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream,
+                   const int32_t* row_map = nullptr, int row_div = 1, void* save0 = nullptr, void* save1 = nullptr) {
   const bool dense = group_sizes == nullptr;
   const int64_t mtiles = dense ? (rows + GBM - 1) / GBM : max_m_tiles(rows, E, GBM);
   const int64_t nt = (N + GBN - 1) / GBN;
   if (mtiles * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
   grouped_gemm_generic_kernel<T, kDual><<<(unsigned)(mtiles * nt), 256, 0, stream>>>(
       static_cast<const T*>(a), static_cast<const T*>(b0), static_cast<const T*>(b1), static_cast<T*>(c), group_sizes,
-      offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)nt);
+      offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)nt, row_map, row_div, static_cast<T*>(save0),
+      static_cast<T*>(save1));
   return JTMOE_OK;
 }
 
 template <typename Cfg>
 int launch_fast(const void* a, const void* b0, const void* b1, void* c, const int32_t* group_sizes,
                 const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream,
-                const int32_t* row_map = nullptr, int row_div = 1, int64_t a_rows = 0) {
+                const int32_t* row_map = nullptr, int row_div = 1, int64_t a_rows = 0, void* save0 = nullptr,
+                void* save1 = nullptr) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   auto kernel = grouped_gemm_dma_kernel<Cfg>;
@@ -165,7 +176,7 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
       static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
       static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,
-      row_map, row_div, (int)a_rows);
+      row_map, row_div, (int)a_rows, static_cast<uint16_t*>(save0), static_cast<uint16_t*>(save1));
   return JTMOE_OK;
 }
 
@@ -183,19 +194,20 @@ template <typename T>
 int launch_pair(const void* x, const void* gate, const void* up, const void* down, const int32_t* group_sizes,
                 const int32_t* offsets, int64_t rows, int64_t H, int64_t I, int64_t E, void* act, void* y,
                 hipStream_t stream, int first_stage, const int32_t* row_map = nullptr, int row_div = 1,
-                int64_t x_rows = 0) {
+                int64_t x_rows = 0, void* save_gate = nullptr, void* save_up = nullptr) {
   if (rows == 0) return JTMOE_OK;
   int rc;
   const bool small = small_groups(rows, E);
-  if (Elem<T>::is_bf16 && fast_ok(x, gate, up, act, H, I))
+  const bool gather_ok = row_map == nullptr || x_rows * H < ((int64_t)1 << 30);
+  const bool saves_ok = save_gate == nullptr || (aligned16(save_gate) && aligned16(save_up));
+  if (Elem<T>::is_bf16 && fast_ok(x, gate, up, act, H, I) && gather_ok && saves_ok)
     rc = small ? launch_fast<GateUpSmallCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
-                                             row_div, x_rows)
+                                             row_div, x_rows, save_gate, save_up)
                : launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
-                                        row_div, x_rows);
-  else if (row_map != nullptr)
-    return fail(JTMOE_EUNSUPPORTED, "grouped_swiglu_gather: shape or alignment outside the gather-on-load path");
+                                        row_div, x_rows, save_gate, save_up);
   else
-    rc = launch_generic<T, true>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream);
+    rc = launch_generic<T, true>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map, row_div,
+                                 save_gate, save_up);
   if (rc) return rc;
   stage_mark(first_stage, stream);
   if (Elem<T>::is_bf16 && fast_ok(act, down, nullptr, y, I, H))
@@ -277,4 +289,48 @@ extern "C" int jtmoe_grouped_swiglu_gather(const void* x, const int32_t* source_
                 "(use jtmoe_dispatch + jtmoe_grouped_swiglu otherwise)");
   return launch_pair<bf16_raw>(x, gate, up, down, group_sizes, offsets, A, H, I, E, act, packed_y, as_stream(stream),
                                kStageGateUp, source_order, (int)K, T);
+}
+
+// Forward pass that keeps what the backward pass needs: the two rounded products
+// gate_pre = round(X Wg[e]) and up_pre = round(X Wu[e]) are stored next to act and packed_y.
+// With source_order the rows of x are fetched through the permutation (packed row j is token
+// source_order[j] / K); without it x is already packed and has T rows.
+extern "C" int jtmoe_grouped_swiglu_train(const void* x, const int32_t* source_order, const void* gate, const void* up,
+                                          const void* down, const int32_t* group_sizes, const int32_t* offsets,
+                                          int64_t T, int64_t K, int64_t H, int64_t I, int64_t E, int dtype,
+                                          void* gate_pre, void* up_pre, void* act, void* packed_y, void* stream) {
+  clear_error();
+  JT_REQUIRE(T >= 0 && K > 0 && T * K < ((int64_t)1 << 31), "grouped_swiglu_train: T=%lld K=%lld out of range",
+             (long long)T, (long long)K);
+  const int64_t A = source_order ? T * K : T;
+  int rc = validate_gemm("grouped_swiglu_train", A, H, I, E, dtype);
+  if (rc) return rc;
+  if (E > JTMOE_MAX_EXPERTS)
+    return fail(JTMOE_EUNSUPPORTED, "grouped_swiglu_train: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  if (A == 0) return JTMOE_OK;
+  JT_REQUIRE(x && gate && up && down && group_sizes && offsets && gate_pre && up_pre && act && packed_y,
+             "grouped_swiglu_train: null pointer argument");
+  hipStream_t s = as_stream(stream);
+  if (dtype == JTMOE_BF16)
+    return launch_pair<bf16_raw>(x, gate, up, down, group_sizes, offsets, A, H, I, E, act, packed_y, s, kStageGateUp,
+                                 source_order, (int)K, T, gate_pre, up_pre);
+  return launch_pair<float>(x, gate, up, down, group_sizes, offsets, A, H, I, E, act, packed_y, s, kStageGateUp,
+                            source_order, (int)K, T, gate_pre, up_pre);
+}
+
+extern "C" int jtmoe_shared_swiglu_train(const void* x, const void* gate, const void* up, const void* down, int64_t T,
+                                         int64_t H, int64_t Is, int dtype, void* gate_pre, void* up_pre, void* act,
+                                         void* shared_y, void* stream) {
+  clear_error();
+  int rc = validate_gemm("shared_swiglu_train", T, H, Is, 1, dtype);
+  if (rc) return rc;
+  if (T == 0) return JTMOE_OK;
+  JT_REQUIRE(x && gate && up && down && gate_pre && up_pre && act && shared_y,
+             "shared_swiglu_train: null pointer argument");
+  hipStream_t s = as_stream(stream);
+  if (dtype == JTMOE_BF16)
+    return launch_pair<bf16_raw>(x, gate, up, down, nullptr, nullptr, T, H, Is, 1, act, shared_y, s,
+                                 kStageSharedGateUp, nullptr, 1, 0, gate_pre, up_pre);
+  return launch_pair<float>(x, gate, up, down, nullptr, nullptr, T, H, Is, 1, act, shared_y, s, kStageSharedGateUp,
+                            nullptr, 1, 0, gate_pre, up_pre);
 }

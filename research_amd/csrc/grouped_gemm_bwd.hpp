@@ -1,0 +1,439 @@
+// The two grouped GEMM forms the backward pass of the expert FFN needs, built from
+// the same parts as grouped_gemm_dma.hpp (tiles written into LDS by
+// buffer_load ... lds, two stages, v_mfma_f32_32x32x16_bf16):
+//
+//   "NT"  C[rows of group e, :] = sum over segments s of  A_s[rows of e, :] @ B_s[e]^T
+//         B_s[e] is [N, K] row-major, i.e. an expert matrix exactly as the forward
+//         pass stores it, used transposed (the data gradient of y = x W is dy W^T).
+//         Both operands are k-contiguous, so both tiles use the row layout with the
+//         XOR swizzle and are read with ds_read_b128.
+//
+//   "TN"  C_i[e] = P[rows of group e, :]^T @ D_i[rows of group e, :]        (i = 0, 1)
+//         one [KA, N] matrix per group, reduced over the rows of the group (the weight
+//         gradient of y = x W is x^T dy).  Both operands are row-major with the
+//         reduction index as the row, so both tiles use the 4 x 16 block layout and are
+//         read with the transposing ds_read_b64_tr_b16.  An empty group yields zeros.
+//
+// Either kernel can fetch operand rows through a row map (packed row j reads row
+// row_map[j] / row_div), the way the forward gate/up launch does, so neither the
+// permuted activations nor the permuted output gradient are ever written to memory.
+//
+// Requirements: bf16, K % 64 == 0 (NT), row lengths multiples of 8, 16-byte aligned
+// pointers, every operand smaller than 2 GiB.
+#pragma once
+
+#include "grouped_gemm_dma.hpp"
+
+namespace jtmoe {
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int OPT_ = 16>
+struct NtGemmCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = 64, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, OPT = OPT_;
+  static constexpr int NT = WAVES_M * WAVES_N * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int A_LOADS = BM * 8 / NT, B_LOADS = BN * 8 / NT;
+  static constexpr int CS = WN + 8;
+  static constexpr size_t EPI_BYTES = (size_t)WAVES_M * WAVES_N * WM * CS * 2;
+  static constexpr size_t PIPE_BYTES = 2 * (size_t)STAGE_BYTES;
+  static constexpr size_t SMEM_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
+  static constexpr int GROUP_M = 4;
+  static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "tiles must divide evenly over the threads");
+  static_assert((NT / 8) % 16 == 0, "swizzle must not depend on the load index");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32x16 MFMAs");
+  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
+};
+
+// A0/A1: [rows, Kdim] (or [a_rows, Kdim] fetched through row_map); B0/B1: [E, N, Kdim];
+// C: [rows, N].  segs = 1 uses A0/B0 only; segs = 2 adds A1 @ B1^T into the same output.
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
+    const uint16_t* __restrict__ A0, const uint16_t* __restrict__ A1, const uint16_t* __restrict__ B0,
+    const uint16_t* __restrict__ B1, uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes,
+    const int32_t* __restrict__ offsets, int E, int dense_rows, int Kdim, int N, int mtiles, int ntiles_n,
+    const int32_t* __restrict__ row_map, int row_div, int a_rows, int segs) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+
+  const int total = mtiles * ntiles_n;
+  const int per_xcd = (int)gridDim.x >> 3;
+  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (logical >= total) return;
+  const int group_span = Cfg::GROUP_M * ntiles_n;
+  const int group = logical / group_span;
+  const int in_group = logical - group * group_span;
+  const int gm = min(Cfg::GROUP_M, mtiles - group * Cfg::GROUP_M);
+  const int nt = in_group / gm;
+  const int mt = group * Cfg::GROUP_M + (in_group - nt * gm);
+
+  TileRows tr = find_tile_wave(mt, BM, group_sizes, offsets, E, dense_rows);
+  tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
+  tr.row0 = __builtin_amdgcn_readfirstlane(tr.row0);
+  tr.rows = __builtin_amdgcn_readfirstlane(tr.rows);
+  if (tr.rows <= 0) return;
+  const int n0 = nt * BN;
+  const size_t wofs = (size_t)tr.expert * Kdim * N;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WAVES_N, wn = wave - wm * Cfg::WAVES_N;
+
+  const bool gather = row_map != nullptr;
+  i32x4_t a_rsrc[2], b_rsrc[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const uint16_t* a = s ? A1 : A0;
+    const uint16_t* b = s ? B1 : B0;
+    if (s >= segs) {
+      a = A0;
+      b = B0;
+    }
+    a_rsrc[s] = gather ? make_rsrc(a, a_rows * Kdim * 2) : make_rsrc(a + (size_t)tr.row0 * Kdim, tr.rows * Kdim * 2);
+    // rows of B past N lie outside the descriptor and read as zeros
+    b_rsrc[s] = make_rsrc(b + wofs, N * Kdim * 2);
+  }
+  // both tiles: slot s = j*NT + tid -> row s/8, slot-in-row s%8 holds source chunk (s%8) ^ ((row/2)%8)
+  const int l_r = tid >> 3, l_slot = tid & 7;
+  const int l_c = l_slot ^ ((l_r >> 1) & 7);
+  int a_voff[Cfg::A_LOADS];
+#pragma unroll
+  for (int j = 0; j < Cfg::A_LOADS; ++j) {
+    const int r = l_r + j * (NT / 8);
+    if (gather)
+      a_voff[j] = r < tr.rows ? ((row_map[tr.row0 + r] / row_div) * Kdim + l_c * 8) * 2 : 0x70000000;
+    else
+      a_voff[j] = (r * Kdim + l_c * 8) * 2;
+  }
+  const int b_voff = ((n0 + l_r) * Kdim + l_c * 8) * 2;
+  const unsigned lds0 = lds_byte_addr(smem_raw);
+  const unsigned wave_lds = lds0 + wave * 1024;
+  const int nk1 = Kdim / BK;
+  const int nk = nk1 * segs;
+
+  auto issue = [&](int kt) {
+    const unsigned base = wave_lds + (kt & 1) * Cfg::STAGE_BYTES;
+    const bool second = kt >= nk1;
+    const int k0 = (second ? kt - nk1 : kt) * BK;
+    const i32x4_t ar = second ? a_rsrc[1] : a_rsrc[0];
+    const i32x4_t br = second ? b_rsrc[1] : b_rsrc[0];
+#pragma unroll
+    for (int j = 0; j < Cfg::A_LOADS; ++j) buffer_load_lds16(ar, base + j * NT * 16, a_voff[j], k0 * 2);
+#pragma unroll
+    for (int j = 0; j < Cfg::B_LOADS; ++j)
+      buffer_load_lds16(br, base + Cfg::A_BYTES + j * NT * 16, b_voff + j * (NT / 8) * Kdim * 2, k0 * 2);
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
+
+  const int sw = ((lane & 31) >> 1) & 7;
+  const int a_rowoff = (wm * WM + (lane & 31)) * (BK * 2);
+  const int b_rowoff = Cfg::A_BYTES + (wn * WN + (lane & 31)) * (BK * 2);
+
+  auto load_frags = [&](const unsigned char* st, int kk, bf16x8_t* af, bf16x8_t* bf) {
+    const int chunk = ((kk * 2 + (lane >> 5)) ^ sw) << 4;
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi)
+      af[mi] = *reinterpret_cast<const bf16x8_t*>(st + a_rowoff + mi * 32 * BK * 2 + chunk);
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj)
+      bf[jj] = *reinterpret_cast<const bf16x8_t*>(st + b_rowoff + jj * 32 * BK * 2 + chunk);
+  };
+
+  if (nk > 0) issue(0);
+  for (int kt = 0; kt < nk; ++kt) {
+    wait_vmcnt<0>();
+    __syncthreads();
+    if (kt + 1 < nk) issue(kt + 1);
+    const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
+    bf16x8_t af[2][TM], bf[2][TN];
+    load_frags(st, 0, af[0], bf[0]);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+#pragma unroll
+      for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj)
+          acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
+      if (Cfg::OPT & 64) {
+#pragma unroll
+        for (int g = 0; g < TM * TN; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+        }
+      }
+    }
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  // epilogue: each wave parks its WM x WN block in its own slice of the idle LDS and streams it
+  // out row by row with 16-byte stores
+  constexpr int CS = Cfg::CS;
+  uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
+#pragma unroll
+  for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+        cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj][i]);
+      }
+  constexpr int CPR_OUT = WN / 8;
+  constexpr int OUT_CHUNKS = WM * CPR_OUT;
+  const int col0 = n0 + wn * WN;
+  const int row_base = wm * WM;
+#pragma unroll
+  for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
+    const int c = lane + j * 64;
+    const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
+    const int col = col0 + ch * 8;
+    if (row_base + r < tr.rows && col < N)
+      *reinterpret_cast<u32x4_t*>(C + (size_t)(tr.row0 + row_base + r) * N + col) = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+
+template <int BMO_, int BNO_, int WAVES_M_, int WAVES_N_, bool kDual_, int OPT_ = 16>
+struct TnGemmCfg {
+  static constexpr int BMO = BMO_, BNO = BNO_, BK = 64, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, OPT = OPT_;
+  static constexpr bool kDual = kDual_;
+  static constexpr int BNE = kDual ? 2 * BNO : BNO;
+  static constexpr int PSUB = BMO / 128, DSUB = BNE / 128;  // 128-column sub-tiles of the two operands
+  static constexpr int NT = WAVES_M * WAVES_N * 64;
+  static constexpr int WM = BMO / WAVES_M, WN = BNE / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int TNO = kDual ? TN / 2 : TN;
+  static constexpr int WNO = TNO * 32;
+  static constexpr int SUB_BYTES = BK * 256;
+  static constexpr int P_BYTES = PSUB * SUB_BYTES;
+  static constexpr int STAGE_BYTES = (PSUB + DSUB) * SUB_BYTES;
+  static constexpr int SUB_LOADS = BK * 16 / NT;
+  static constexpr int CS = WNO + 8;
+  static constexpr size_t EPI_BYTES = (size_t)WAVES_M * WAVES_N * WM * CS * 2;
+  static constexpr size_t PIPE_BYTES = 2 * (size_t)STAGE_BYTES;
+  static constexpr size_t SMEM_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
+  static_assert(BMO % 128 == 0 && BNE % 128 == 0, "operand tiles are made of 128-column sub-tiles");
+  static_assert((BK * 16) % NT == 0, "sub-tile must divide evenly over the threads");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32x16 MFMAs");
+  static_assert(!kDual || (TN % 2 == 0 && BNO == 128), "dual tiles: one sub-tile per matrix");
+  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
+};
+
+// P: [rows, KA] (or [p_rows, KA] through row_map when p_gather); D0/D1: [rows, N] (or [d_rows, N]
+// through row_map when d_gather); C0/C1: [E, KA, N].
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
+    const uint16_t* __restrict__ P, const uint16_t* __restrict__ D0, const uint16_t* __restrict__ D1,
+    uint16_t* __restrict__ C0, uint16_t* __restrict__ C1, const int32_t* __restrict__ group_sizes,
+    const int32_t* __restrict__ offsets, int E, int dense_rows, int KA, int N, int mtiles_o, int ntiles_o,
+    const int32_t* __restrict__ row_map, int row_div, int p_gather, int d_gather, int gathered_rows) {
+  constexpr int BMO = Cfg::BMO, BNO = Cfg::BNO, BK = Cfg::BK, NT = Cfg::NT;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
+  constexpr bool kDual = Cfg::kDual;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+
+  // consecutive workgroup ids go round-robin to the 8 XCDs: give each XCD a contiguous range of
+  // (group, tile) pairs so that all tiles of one group read its rows through the same L2
+  const int per_group = mtiles_o * ntiles_o;
+  const int total = E * per_group;
+  const int per_xcd = (int)gridDim.x >> 3;
+  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (logical >= total) return;
+  const int e = logical / per_group;
+  const int in_e = logical - e * per_group;
+  const int nt = in_e / mtiles_o;
+  const int mt = in_e - nt * mtiles_o;
+  const int m0 = mt * BMO, n0 = nt * BNO;
+
+  int row0, rows;
+  if (group_sizes) {
+    row0 = __builtin_amdgcn_readfirstlane(offsets[e]);
+    rows = __builtin_amdgcn_readfirstlane(group_sizes[e]);
+  } else {
+    row0 = 0;
+    rows = dense_rows;
+  }
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WAVES_N, wn = wave - wm * Cfg::WAVES_N;
+
+  const i32x4_t p_rsrc = p_gather ? make_rsrc(P, gathered_rows * KA * 2)
+                                  : make_rsrc(P + (size_t)row0 * KA, rows * KA * 2);
+  i32x4_t d_rsrc[Cfg::DSUB];
+#pragma unroll
+  for (int u = 0; u < Cfg::DSUB; ++u) {
+    const uint16_t* d = (kDual && u == 1) ? D1 : D0;
+    d_rsrc[u] = d_gather ? make_rsrc(d, gathered_rows * N * 2) : make_rsrc(d + (size_t)row0 * N, rows * N * 2);
+  }
+  // sub-tile [BK rows][128 columns] as 128-byte blocks of 4 rows x 16 columns, block (r/4, c/16) at
+  // index (r/4)*8 + c/16; slot s (16 bytes) -> block s/8, row (s/2)%4 of the block, half s%2
+  // (OPT & 128: 512-byte blocks of 4 rows x 64 columns instead, block (r/4, c/64) at index
+  // (r/4)*2 + c/64, so that eight lanes fetch one whole 128-byte line)
+  constexpr bool kWide = (Cfg::OPT & 128) != 0;
+  const int b_blk_id = kWide ? tid >> 5 : tid >> 3;
+  // row inside the k step (first load) and 16-byte chunk inside the 128 columns
+  const int l_r = kWide ? (b_blk_id >> 1) * 4 + ((tid >> 3) & 3) : (b_blk_id >> 3) * 4 + ((tid >> 1) & 3);
+  const int l_c = kWide ? (b_blk_id & 1) * 8 + (tid & 7) : (b_blk_id & 7) * 2 + (tid & 1);
+  constexpr int ROWS_PER_LOAD = NT / 16;
+  const int p_col = (m0 + l_c * 8) * 2, d_col = (n0 + l_c * 8) * 2;  // byte offset inside a row
+  const unsigned lds0 = lds_byte_addr(smem_raw);
+  const unsigned wave_lds = lds0 + wave * 1024;
+  const int nk = (rows + BK - 1) / BK;
+
+  // row ids of a k step (only used by gathered operands); -1 = past the end of the group
+  int ids[Cfg::SUB_LOADS];
+  auto fetch_ids = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < Cfg::SUB_LOADS; ++j) {
+      const int r = kt * BK + l_r + j * ROWS_PER_LOAD;
+      ids[j] = r < rows ? row_map[row0 + r] / row_div : -1;
+    }
+  };
+  const bool any_gather = p_gather || d_gather;
+  if (any_gather && nk > 0) fetch_ids(0);
+
+  // Rows past the end of the group must contribute zeros: their offsets lie outside the
+  // descriptor (which ends with the group, or is pushed there explicitly for gathered rows).
+  auto issue = [&](int kt) {
+    const unsigned base = wave_lds + (kt & 1) * Cfg::STAGE_BYTES;
+    int pv[Cfg::SUB_LOADS], dv[Cfg::SUB_LOADS];
+#pragma unroll
+    for (int j = 0; j < Cfg::SUB_LOADS; ++j) {
+      const int r = kt * BK + l_r + j * ROWS_PER_LOAD;
+      pv[j] = p_gather ? (ids[j] >= 0 ? ids[j] * KA * 2 + p_col : 0x70000000) : r * KA * 2 + p_col;
+      dv[j] = d_gather ? (ids[j] >= 0 ? ids[j] * N * 2 + d_col : 0x70000000) : r * N * 2 + d_col;
+    }
+#pragma unroll
+    for (int u = 0; u < Cfg::PSUB; ++u)
+#pragma unroll
+      for (int j = 0; j < Cfg::SUB_LOADS; ++j)
+        buffer_load_lds16(p_rsrc, base + u * Cfg::SUB_BYTES + j * NT * 16, pv[j] + u * 256, 0);
+#pragma unroll
+    for (int u = 0; u < Cfg::DSUB; ++u)
+#pragma unroll
+      for (int j = 0; j < Cfg::SUB_LOADS; ++j)
+        buffer_load_lds16(d_rsrc[u], base + Cfg::P_BYTES + u * Cfg::SUB_BYTES + j * NT * 16,
+                          dv[j] + (kDual ? 0 : u * 256), 0);
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
+
+  // transposing read: the 16 lanes of a group read one whole 128-byte block, lane i its bytes
+  // [8 i, 8 i + 8) = row i/4, columns 4*(i%4)..; groups: column half (lane/16)%2, row half lane/32
+  const int laneoff = kWide ? ((lane & 15) >> 2) * 128 + (lane & 3) * 8 + ((lane >> 4) & 1) * 32 + (lane >> 5) * 2048
+                            : (lane & 15) * 8 + ((lane >> 4) & 1) * 128 + (lane >> 5) * (2 * 8 * 128);
+  auto block_of = [&](int col) {
+    return kWide ? (col >> 7) * Cfg::SUB_BYTES + ((col & 127) >> 6) * 512 + (col & 63) * 2
+                 : (col >> 7) * Cfg::SUB_BYTES + ((col & 127) >> 4) * 128;
+  };
+  int p_blk[TM], d_blk[TN];
+#pragma unroll
+  for (int mi = 0; mi < TM; ++mi) p_blk[mi] = block_of(wm * WM + mi * 32);
+#pragma unroll
+  for (int jj = 0; jj < TN; ++jj) {
+    int col;
+    if (kDual)
+      col = (jj < TN / 2 ? 0 : BNO) + wn * (WN / 2) + (jj % (TN / 2)) * 32;
+    else
+      col = wn * WN + jj * 32;
+    d_blk[jj] = Cfg::P_BYTES + block_of(col);
+  }
+  auto read_tr = [&](const unsigned char* p) {
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+    const s16x4_t hi =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 8 * 128));
+    const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8_t, both);
+  };
+  auto load_frags = [&](const unsigned char* st, int kk, bf16x8_t* af, bf16x8_t* bf) {
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi) af[mi] = read_tr(st + p_blk[mi] + laneoff + kk * (4 * 8 * 128));
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj) bf[jj] = read_tr(st + d_blk[jj] + laneoff + kk * (4 * 8 * 128));
+  };
+
+  if (nk > 0) {
+    issue(0);
+    if (any_gather && nk > 1) fetch_ids(1);
+  }
+  for (int kt = 0; kt < nk; ++kt) {
+    wait_vmcnt<0>();
+    __syncthreads();
+    if (kt + 1 < nk) {
+      issue(kt + 1);
+      if (any_gather && kt + 2 < nk) fetch_ids(kt + 2);
+    }
+    const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
+    bf16x8_t af[2][TM], bf[2][TN];
+    load_frags(st, 0, af[0], bf[0]);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+#pragma unroll
+      for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj)
+          acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
+    }
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  // epilogue: per matrix, each wave parks its WM x WNO block in LDS and streams it out in rows
+  constexpr int TNO = Cfg::TNO, WNO = Cfg::WNO, CS = Cfg::CS;
+  uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
+  constexpr int CPR_OUT = WNO / 8;
+  constexpr int OUT_CHUNKS = WM * CPR_OUT;
+  const int col0 = n0 + wn * WNO;
+  const int row_base = m0 + wm * WM;
+#pragma unroll
+  for (int which = 0; which < (kDual ? 2 : 1); ++which) {
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+      for (int jj = 0; jj < TNO; ++jj)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+          cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj + which * (TN / 2)][i]);
+        }
+    uint16_t* const Cm = (which ? C1 : C0) + (size_t)e * KA * N;
+#pragma unroll
+    for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
+      const int c = lane + j * 64;
+      const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
+      const int col = col0 + ch * 8;
+      if (row_base + r < KA && col < N) *reinterpret_cast<u32x4_t*>(Cm + (size_t)(row_base + r) * N + col) = v;
+    }
+    // the staging area is private to the wave and the second matrix is written by the same
+    // lanes' LDS stores after their loads above: program order within the wave suffices
+  }
+}
+
+// Configurations the library launches.
+using DgradCfg = NtGemmCfg<256, 256, 2, 4, 16 + 64>;   // data gradients: 256 x 256 tiles
+using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16 + 128>;  // gate and up weight gradients share the x tile
+using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16 + 128>;     // down weight gradient
+
+}  // namespace jtmoe

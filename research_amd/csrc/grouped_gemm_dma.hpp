@@ -109,7 +109,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
     uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
     int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
-    int a_rows) {
+    int a_rows, uint16_t* __restrict__ save0 = nullptr, uint16_t* __restrict__ save1 = nullptr) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, NSTAGE = Cfg::NSTAGE;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   constexpr int CPRA = Cfg::CPRA;
@@ -291,39 +291,45 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   // Value i of lane l in a 32x32 accumulator is row 8*(i/4) + 4*(l/32) + i%4, column l%32: a
   // lane holds single elements of many rows.  Each wave parks its WM x WNO block of results
   // in its own slice of the idle LDS and streams it out row by row with 16-byte stores.
+  // With save0 / save1 (dual tiles only) the two rounded products themselves, which the backward
+  // pass needs, are written as well: pass 0 stores the result, passes 1 and 2 the two products.
   constexpr int TNO = Cfg::TNO, WNO = Cfg::WNO, CS = Cfg::CS;
   uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
-#pragma unroll
-  for (int mi = 0; mi < TM; ++mi) {
-#pragma unroll
-    for (int jj = 0; jj < TNO; ++jj) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-        float v;
-        if (kDual) {
-          const float g = bf16_round_fast(acc[mi][jj][i]);
-          const float u = bf16_round_fast(acc[mi][jj + TN / 2][i]);
-          v = silu_rcp(g) * u;
-        } else {
-          v = acc[mi][jj][i];
-        }
-        cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(v);
-      }
-    }
-  }
   constexpr int CPR_OUT = WNO / 8;
   constexpr int OUT_CHUNKS = WM * CPR_OUT;
   const int col0 = n0 + wn * WNO;
   const int row_base = wm * WM;
+  const int passes = (kDual && save0 != nullptr) ? 3 : 1;
+  for (int pass = 0; pass < passes; ++pass) {
 #pragma unroll
-  for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
-    const int c = lane + j * 64;
-    const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
-    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
-    const int col = col0 + ch * 8;
-    if (row_base + r < tr.rows && col < N)
-      *reinterpret_cast<u32x4_t*>(C + (size_t)(tr.row0 + row_base + r) * N + col) = v;
+    for (int mi = 0; mi < TM; ++mi) {
+#pragma unroll
+      for (int jj = 0; jj < TNO; ++jj) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+          float v;
+          if (kDual) {
+            const float g = bf16_round_fast(acc[mi][jj][i]);
+            const float u = bf16_round_fast(acc[mi][jj + TN / 2][i]);
+            v = pass == 0 ? silu_rcp(g) * u : (pass == 1 ? g : u);
+          } else {
+            v = acc[mi][jj][i];
+          }
+          cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(v);
+        }
+      }
+    }
+    uint16_t* const out = pass == 0 ? C : (pass == 1 ? save0 : save1);
+#pragma unroll
+    for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
+      const int c = lane + j * 64;
+      const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
+      const int col = col0 + ch * 8;
+      if (row_base + r < tr.rows && col < N)
+        *reinterpret_cast<u32x4_t*>(out + (size_t)(tr.row0 + row_base + r) * N + col) = v;
+    }
   }
 }
 

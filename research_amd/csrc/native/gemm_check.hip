@@ -4,9 +4,10 @@
 // accumulation in k order), a tolerance, and PASS / FAIL on stdout.
 //
 //   gemm_check            correctness on ragged groups, gather-on-load and the dense case
+//   gemm_check time_backward   + timing of the four backward launches at the C3 shape
 //   gemm_check time       + timing of the library's two configurations at the C3 shape,
 //                           once on N(0,1)-like data and once on all-zero data
-#include "grouped_gemm_dma.hpp"
+#include "grouped_gemm_bwd.hpp"
 
 #include <cmath>
 #include <cstdio>
@@ -128,7 +129,7 @@ static void launch(Problem& p, bool dense) {
   const long nt = (p.N + Cfg::BN - 1) / Cfg::BN;
   kernel<<<(unsigned)gemm_grid(mt, nt), Cfg::NT, Cfg::SMEM_BYTES>>>(
       p.A, p.B0, Cfg::kDual ? p.B1 : nullptr, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows,
-      p.K, p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows);
+      p.K, p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, nullptr, nullptr);
 }
 
 template <typename Cfg>
@@ -177,6 +178,209 @@ static void timeit(const char* name, Problem& p, int iters) {
   fflush(stdout);
 }
 
+// ---- the two backward forms -------------------------------------------------------------------
+
+// C[r, n] = sum_s sum_k A_s[arow(r), k] * B_s[e(r), n, k]
+__global__ void reference_nt_kernel(const uint16_t* A0, const uint16_t* A1, const uint16_t* B0, const uint16_t* B1,
+                                    float* C, const int* row_expert, const int* a_row_of, int rows, int K, int N,
+                                    int segs) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (n >= N || r >= rows) return;
+  const int e = row_expert[r];
+  float acc = 0;
+  for (int s = 0; s < segs; ++s) {
+    const uint16_t* a = (s ? A1 : A0) + (size_t)a_row_of[r] * K;
+    const uint16_t* b = (s ? B1 : B0) + ((size_t)e * N + n) * K;
+    for (int k = 0; k < K; ++k) acc += bf16_bits_to_f32(a[k]) * bf16_bits_to_f32(b[k]);
+  }
+  C[(size_t)r * N + n] = acc;
+}
+
+// C[e, ka, n] = sum over rows r of group e of P[prow(r), ka] * D[drow(r), n]
+__global__ void reference_tn_kernel(const uint16_t* P, const uint16_t* D, float* C, const int* gs, const int* off,
+                                    const int* p_row_of, const int* d_row_of, int KA, int N) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x, ka = blockIdx.y, e = blockIdx.z;
+  if (n >= N) return;
+  float acc = 0;
+  for (int r = off[e]; r < off[e] + gs[e]; ++r)
+    acc += bf16_bits_to_f32(P[(size_t)p_row_of[r] * KA + ka]) * bf16_bits_to_f32(D[(size_t)d_row_of[r] * N + n]);
+  C[((size_t)e * KA + ka) * N + n] = acc;
+}
+
+static uint16_t* random_bf16(size_t n, unsigned seed, float scale) {
+  std::vector<uint16_t> h(n);
+  std::mt19937 rng(seed);
+  std::normal_distribution<float> nd(0.f, 1.f);
+  for (auto& v : h) v = f2bf(nd(rng) * scale);
+  uint16_t* d;
+  CK(hipMalloc(&d, n * 2));
+  CK(hipMemcpy(d, h.data(), n * 2, hipMemcpyHostToDevice));
+  return d;
+}
+
+static bool compare(const char* name, const float* dref, const uint16_t* dgot, size_t n, const char* shape) {
+  std::vector<float> hr(n);
+  std::vector<uint16_t> hc(n);
+  CK(hipMemcpy(hr.data(), dref, n * 4, hipMemcpyDeviceToHost));
+  CK(hipMemcpy(hc.data(), dgot, n * 2, hipMemcpyDeviceToHost));
+  double maxref = 0, maxerr = 0;
+  size_t bad = 0;
+  for (float v : hr) maxref = std::max(maxref, (double)std::fabs(v));
+  for (size_t i = 0; i < n; ++i) {
+    const double e = std::fabs((double)bf2f(hc[i]) - hr[i]);
+    if (!(e <= 0.02 * maxref)) ++bad;
+    maxerr = std::max(maxerr, e);
+  }
+  printf("case %-34s %s max_err/max_ref=%.3e tolerance=2e-2 bad=%zu\n", name, shape, maxerr / maxref, bad);
+  fflush(stdout);
+  return bad == 0;
+}
+
+template <typename Cfg>
+static void launch_nt(Problem& p, const uint16_t* A1, int segs, bool dense) {
+  auto kernel = grouped_gemm_nt_kernel<Cfg>;
+  CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                         (int)Cfg::SMEM_BYTES));
+  const long mt = dense ? (p.rows + Cfg::BM - 1) / Cfg::BM
+                        : (p.rows + Cfg::BM - 1) / Cfg::BM + (p.E < p.rows ? p.E : p.rows);
+  const long nt = (p.N + Cfg::BN - 1) / Cfg::BN;
+  kernel<<<(unsigned)gemm_grid(mt, nt), Cfg::NT, Cfg::SMEM_BYTES>>>(
+      p.A, A1, p.B0, p.B1, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows, p.K, p.N, (int)mt,
+      (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, segs);
+}
+
+// B0 / B1 of the problem are read as [E, N, K] here
+template <typename Cfg>
+static bool check_nt(const char* name, Problem& p, int segs, bool dense = false) {
+  uint16_t* A1 = segs == 2 ? random_bf16((size_t)p.a_rows * p.K, 77, 1.0f) : nullptr;
+  float* ref;
+  CK(hipMalloc(&ref, (size_t)p.rows * p.N * 4));
+  reference_nt_kernel<<<dim3((p.N + 255) / 256, p.rows), 256>>>(p.A, A1, p.B0, p.B1, ref, p.drow, p.darow, p.rows,
+                                                               p.K, p.N, segs);
+  CK(hipMemset(p.C, 0xff, (size_t)p.rows * p.N * 2));
+  launch_nt<Cfg>(p, A1, segs, dense);
+  CK(hipDeviceSynchronize());
+  char shape[128];
+  snprintf(shape, sizeof shape, "E=%d rows=%d K=%d N=%d segs=%d", p.E, p.rows, p.K, p.N, segs);
+  const bool ok = compare(name, ref, p.C, (size_t)p.rows * p.N, shape);
+  hipFree(ref);
+  if (A1) hipFree(A1);
+  return ok;
+}
+
+template <typename Cfg>
+static void launch_tn(Problem& p, const uint16_t* D0, const uint16_t* D1, uint16_t* C0, uint16_t* C1, bool p_gather,
+                      bool d_gather, bool dense) {
+  auto kernel = grouped_gemm_tn_kernel<Cfg>;
+  CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                         (int)Cfg::SMEM_BYTES));
+  const long mt = (p.K + Cfg::BMO - 1) / Cfg::BMO, nt = (p.N + Cfg::BNO - 1) / Cfg::BNO;
+  const int groups = dense ? 1 : p.E;
+  kernel<<<(unsigned)gemm_grid(groups * mt, nt), Cfg::NT, Cfg::SMEM_BYTES>>>(
+      p.A, D0, D1, C0, C1, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, groups, p.rows, p.K, p.N, (int)mt,
+      (int)nt, p.dmap, p.top_k > 0 ? p.top_k : 1, p_gather, d_gather, p.a_rows);
+}
+
+// which operand goes through the row map: 0 none, 1 the transposed one (P), 2 the other (D)
+template <typename Cfg>
+static bool check_tn(const char* name, Problem& p, int gather_which, bool dense = false) {
+  const bool pg = gather_which == 1, dg = gather_which == 2;
+  // P is p.A ([a_rows, K] if gathered, else its first rows are used as [rows, K]: make sure it is big enough)
+  uint16_t* P = pg ? p.A : random_bf16((size_t)p.rows * p.K, 91, 1.0f);
+  const size_t d_rows = dg ? p.a_rows : p.rows;
+  uint16_t* D0 = random_bf16(d_rows * p.N, 92, 1.0f);
+  uint16_t* D1 = random_bf16(d_rows * p.N, 93, 1.0f);
+  const size_t out = (size_t)(dense ? 1 : p.E) * p.K * p.N;
+  uint16_t *C0, *C1;
+  CK(hipMalloc(&C0, out * 2)); CK(hipMalloc(&C1, out * 2));
+  CK(hipMemset(C0, 0xff, out * 2)); CK(hipMemset(C1, 0xff, out * 2));
+  // identity row lookup for operands that are not gathered
+  std::vector<int> ident(p.rows);
+  for (int r = 0; r < p.rows; ++r) ident[r] = r;
+  int* dident;
+  CK(hipMalloc(&dident, p.rows * 4));
+  CK(hipMemcpy(dident, ident.data(), p.rows * 4, hipMemcpyHostToDevice));
+  std::vector<int> one_gs{p.rows}, one_off{0};
+  int *dgs1, *doff1;
+  CK(hipMalloc(&dgs1, 4)); CK(hipMalloc(&doff1, 4));
+  CK(hipMemcpy(dgs1, one_gs.data(), 4, hipMemcpyHostToDevice));
+  CK(hipMemcpy(doff1, one_off.data(), 4, hipMemcpyHostToDevice));
+  float *ref0, *ref1;
+  CK(hipMalloc(&ref0, out * 4)); CK(hipMalloc(&ref1, out * 4));
+  const dim3 grid((p.N + 255) / 256, p.K, dense ? 1 : p.E);
+  reference_tn_kernel<<<grid, 256>>>(P, D0, ref0, dense ? dgs1 : p.dgs, dense ? doff1 : p.doff, pg ? p.darow : dident,
+                                     dg ? p.darow : dident, p.K, p.N);
+  reference_tn_kernel<<<grid, 256>>>(P, D1, ref1, dense ? dgs1 : p.dgs, dense ? doff1 : p.doff, pg ? p.darow : dident,
+                                     dg ? p.darow : dident, p.K, p.N);
+  Problem q = p;
+  q.A = P;
+  launch_tn<Cfg>(q, D0, D1, C0, C1, pg, dg, dense);
+  CK(hipDeviceSynchronize());
+  char shape[128];
+  snprintf(shape, sizeof shape, "E=%d rows=%d KA=%d N=%d gather=%d", p.E, p.rows, p.K, p.N, gather_which);
+  bool ok = compare(name, ref0, C0, out, shape);
+  if (Cfg::kDual) ok &= compare(name, ref1, C1, out, shape);
+  hipFree(ref0); hipFree(ref1); hipFree(C0); hipFree(C1); hipFree(D0); hipFree(D1); hipFree(dident);
+  hipFree(dgs1); hipFree(doff1);
+  if (!pg) hipFree(P);
+  return ok;
+}
+
+template <typename F>
+static void time_launches(const char* name, double flops, int iters, F launch_once) {
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
+  for (int i = 0; i < 5; ++i) launch_once();
+  CK(hipDeviceSynchronize());
+  CK(hipEventRecord(a));
+  for (int i = 0; i < iters; ++i) launch_once();
+  CK(hipEventRecord(b)); CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= iters;
+  printf("time %-44s %.3f ms  %.1f TFLOP/s  (%.1f%% of 2500)\n", name, ms, flops / ms / 1e9, flops / ms / 1e9 / 25.0);
+  fflush(stdout);
+}
+
+// the four backward launches of the routed experts at the layer shape: 64 groups, 131072 packed
+// rows that are 16384 token rows fetched through a permutation, hidden 2048, intermediate 1408
+static void time_backward() {
+  const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
+  {  // d act = dy[token of row] @ Wd^T : A gathered [T, H], B [E, I, H]
+    Problem p = make(E, rows, H, I, 21, false, topk, 1.0f);
+    time_launches("dgrad down (gathered dy @ Wd^T)", 2.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(p, nullptr, 1, false); });
+    // dWg, dWu = x[token of row]^T @ (dG, dU)
+    uint16_t* D0 = random_bf16((size_t)rows * I, 31, 1.0f);
+    uint16_t* D1 = random_bf16((size_t)rows * I, 32, 1.0f);
+    uint16_t *C0, *C1;
+    CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
+    time_launches("wgrad gate/up (gathered x^T @ dG, dU)", 4.0 * rows * H * I, 10,
+                  [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, true, false, false); });
+    hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1);
+    release(p);
+  }
+  {  // dXp = dG @ Wg^T + dU @ Wu^T : A [rows, I] twice, B [E, H, I] twice
+    Problem p = make(E, rows, I, H, 22, false, 0, 1.0f);
+    uint16_t* A1 = random_bf16((size_t)rows * I, 33, 1.0f);
+    time_launches("dgrad gate/up (dG @ Wg^T + dU @ Wu^T)", 4.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(p, A1, 2, false); });
+    hipFree(A1);
+    release(p);
+  }
+  {  // dWd = (w * act)^T @ dy[token of row] : P [rows, I], D gathered [T, H]
+    Problem p = make(E, rows, I, H, 23, false, topk, 1.0f);  // p.A is [T, I] here and unused as P
+    uint16_t* P = random_bf16((size_t)rows * I, 34, 1.0f);
+    uint16_t* D = random_bf16((size_t)T * H, 35, 1.0f);
+    uint16_t* C0;
+    CK(hipMalloc(&C0, (size_t)E * H * I * 2));
+    Problem q = p;
+    q.A = P;
+    time_launches("wgrad down (act^T @ gathered dy)", 2.0 * rows * H * I, 10,
+                  [&] { launch_tn<WgradCfg>(q, D, nullptr, C0, nullptr, false, true, false); });
+    hipFree(P); hipFree(D); hipFree(C0);
+    release(p);
+  }
+}
+
 int main(int argc, char** argv) {
   bool ok = true;
   {
@@ -207,6 +411,29 @@ int main(int argc, char** argv) {
     ok &= check<GateUpSmallCfg>("gate/up few rows, gather on load", p);
     release(p);
   }
+  {
+    Problem p = make(7, 3001, 576, 392, 11, true, 0, 1.0f);
+    ok &= check_nt<DgradCfg>("dgrad ragged", p, 1);
+    ok &= check_nt<DgradCfg>("dgrad ragged, two segments", p, 2);
+    ok &= check_tn<WgradCfg>("wgrad ragged", p, 0);
+    ok &= check_tn<WgradDualCfg>("wgrad dual ragged", p, 0);
+    release(p);
+  }
+  {
+    Problem p = make(5, 2400, 512, 384, 12, true, 3, 1.0f);
+    ok &= check_nt<DgradCfg>("dgrad gather on load", p, 1);
+    ok &= check_tn<WgradDualCfg>("wgrad dual, transposed operand gathered", p, 1);
+    ok &= check_tn<WgradCfg>("wgrad, other operand gathered", p, 2);
+    release(p);
+  }
+  {
+    Problem p = make(1, 777, 512, 520, 13, false, 0, 1.0f);
+    ok &= check_nt<DgradCfg>("dgrad dense", p, 2, true);
+    ok &= check_tn<WgradCfg>("wgrad dense", p, 0, true);
+    ok &= check_tn<WgradDualCfg>("wgrad dual dense", p, 0, true);
+    release(p);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_backward")) time_backward();
   if (ok && argc > 1 && !strcmp(argv[1], "time")) {
     for (float scale : {1.0f, 0.0f}) {
       printf("-- operand data: %s\n", scale > 0 ? "N(0,1) activations, N(0,0.05) weights" : "all zeros");
@@ -217,6 +444,7 @@ int main(int argc, char** argv) {
       timeit<DownCfg>("down 64 groups", d, 20);
       release(d);
     }
+    time_backward();
     // decode-sized batch: 8 rows per group, bound by streaming the expert matrices
     Problem g = make(64, 512, 2048, 1408, 8, false, 0, 1.0f);
     timeit<GateUpCfg>("gate/up 64 groups, 256-row tiles", g, 20);

@@ -1,0 +1,202 @@
+"""Parity of the backward pass (through the C ABI) with the float64 gradient oracle, on the GPU.
+
+The specification is the reference's own gradient test of the expert dispatcher
+(tests/jaxtitan/test_model.py:549-691): gradients with respect to x, the route weights and the
+three expert matrices on four routing patterns, rtol = atol = 1e-5 in fp32, and bit-identical
+results when the call is repeated.  bf16 results are held to max|g-ref|/max|ref| <= 2e-2 per
+tensor, the bar of the forward pass.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_grad_oracle as G
+from oracle import moe_oracle as O
+from research_amd import grad, ops
+from test_gpu_parity import BF16_MAX_REL, dev, host, random_problem, report
+from test_oracle_grad import reference_case
+
+pytestmark = pytest.mark.gpu
+
+F32_GRAD_TOL = dict(rtol=1e-5, atol=1e-5)
+
+
+def expert_grads(gpu, x, ids, w, gate, up, down, dy, dtype, dx_extra=None):
+    xd, gd, ud, dd, wd, dyd = (dev(a.astype(np.float32), gpu, dtype) for a in (x, gate, up, down, w, dy))
+    plan = ops.dispatch(dev(ids.astype(np.int32), gpu), gate.shape[0])
+    packed_y, act, res = grad.grouped_swiglu_train(xd, plan.source_order, ids.shape[1], gd, ud, dd, plan.group_sizes,
+                                                   plan.offsets)
+    extra = None if dx_extra is None else dev(dx_extra.astype(np.float32), gpu, dtype)
+    return grad.experts_backward(xd, dyd, plan, wd, gd, ud, dd, res, dx_extra=extra), (packed_y, act, res, plan)
+
+
+@pytest.mark.parametrize("pattern", ["balanced", "no_expert_three", "all_one_expert", "duplicate_routes"])
+@pytest.mark.parametrize("batch", [1, 2])
+def test_expert_gradients_on_the_reference_case_fp32(gpu, pattern, batch):
+    x, gate, up, down, weights, patterns, cot = reference_case(batch)
+    ids = patterns[pattern]
+    want = G.experts_backward(x, ids, weights, gate, up, down, cot)
+    got, _ = expert_grads(gpu, x, ids, weights, gate, up, down, cot, "f32")
+    again, _ = expert_grads(gpu, x, ids, weights, gate, up, down, cot, "f32")
+    for name in ("dx", "d_weights", "d_gate", "d_up", "d_down"):
+        g = getattr(got, name)
+        assert bool(torch.isfinite(g).all())
+        np.testing.assert_allclose(host(g), getattr(want, name), err_msg=f"{pattern} {name}", **F32_GRAD_TOL)
+        assert torch.equal(g, getattr(again, name)), f"{name} differs between two identical calls"
+
+
+@pytest.mark.parametrize(
+    "tokens,hidden,experts,top_k,inter,dtype",
+    [(70, 32, 4, 2, 64, "f32"), (200, 192, 8, 2, 320, "f32"), (300, 64, 6, 3, 96, "bf16"), (257, 200, 5, 2, 136, "bf16"),
+     (700, 1024, 16, 2, 704, "bf16"), (512, 2048, 64, 8, 1408, "bf16")],
+)
+def test_expert_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, inter, dtype):
+    std = 0.02 if hidden >= 512 else 0.2
+    x, gate, up, down, ids, w = random_problem(100 + tokens, tokens, hidden, experts, top_k, inter, std)
+    rng = np.random.default_rng(tokens)
+    ids[: tokens // 4] = ids[0]  # skew; leaves some experts with few rows
+    dy = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    extra = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    cast = lambda a: O.cast_compute(a, dtype)
+    want = G.experts_backward(cast(x), ids, cast(w), cast(gate), cast(up), cast(down), cast(dy))
+    got, (packed_y, act, res, plan) = expert_grads(gpu, x, ids, w, gate, up, down, dy, dtype, dx_extra=extra)
+    # the training forward returns what the plain forward returns, and the two products it keeps
+    d = O.dispatch(ids, experts, cast(x))
+    ref_y, ref_g, ref_u, _ = O.grouped_swiglu(d.packed_x, gate, up, down, d.group_sizes, dtype, return_stages=True)
+    plain = ops.grouped_swiglu_gather(dev(x, gpu, dtype), plan.source_order, top_k, dev(gate, gpu, dtype),
+                                      dev(up, gpu, dtype), dev(down, gpu, dtype), plan.group_sizes,
+                                      plan.offsets) if dtype == "bf16" and hidden % 64 == 0 and inter % 64 == 0 else None
+    if plain is not None:
+        assert torch.equal(plain, packed_y)
+    tag = f"grad {dtype} T={tokens} H={hidden} E={experts} K={top_k} I={inter}"
+    wants = dict(dx=want.dx + cast(extra), d_weights=want.d_weights, d_gate=want.d_gate, d_up=want.d_up,
+                 d_down=want.d_down)
+    if dtype == "bf16":
+        assert report(tag + " gate_pre", host(res.gate_pre), ref_g) <= BF16_MAX_REL
+        assert report(tag + " up_pre", host(res.up_pre), ref_u) <= BF16_MAX_REL
+        assert report(tag + " packed_y", host(packed_y), ref_y) <= BF16_MAX_REL
+        for name, ref in wants.items():
+            assert report(f"{tag} {name}", host(getattr(got, name)), ref.astype(np.float32)) <= BF16_MAX_REL
+    else:
+        np.testing.assert_allclose(host(res.gate_pre), ref_g, rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(host(res.up_pre), ref_u, rtol=2e-5, atol=2e-5)
+        for name, ref in wants.items():
+            scale = float(np.max(np.abs(ref))) or 1.0
+            np.testing.assert_allclose(host(getattr(got, name)) / scale, ref / scale, rtol=1e-4, atol=2e-5,
+                                       err_msg=name)
+    # experts that received no row get exactly zero weight gradients
+    for e in np.nonzero(host(plan.group_sizes) == 0)[0]:
+        assert not got.d_gate[e].any() and not got.d_up[e].any() and not got.d_down[e].any()
+
+
+@pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16")])
+def test_shared_gradients_match_oracle(gpu, tokens, hidden, inter, dtype):
+    rng = np.random.default_rng(7)
+    std = 0.02 if hidden >= 512 else 0.2
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    gate, up = (rng.standard_normal((hidden, inter)).astype(np.float32) * std for _ in range(2))
+    down = rng.standard_normal((inter, hidden)).astype(np.float32) * std
+    dy = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    cast = lambda a: O.cast_compute(a, dtype)
+    want = G.shared_backward(cast(x), cast(gate), cast(up), cast(down), cast(dy))
+    xd, gd, ud, dd, dyd = (dev(a, gpu, dtype) for a in (x, gate, up, down, dy))
+    y, res = grad.shared_swiglu_train(xd, gd, ud, dd)
+    assert torch.equal(y, ops.shared_swiglu(xd, gd, ud, dd))
+    got = grad.shared_backward(xd, dyd, gd, ud, dd, res)
+    for name, g, ref in zip(("dx", "d_gate", "d_up", "d_down"), got, (want.dx, want.d_gate, want.d_up, want.d_down)):
+        if dtype == "bf16":
+            assert report(f"shared grad T={tokens} H={hidden} I={inter} {name}", host(g), ref.astype(np.float32)) <= BF16_MAX_REL
+        else:
+            np.testing.assert_allclose(host(g), ref, rtol=1e-4, atol=2e-5, err_msg=name)
+
+
+@pytest.mark.parametrize("tokens,hidden,experts,top_k,dtype,with_scores",
+                         [(6, 5, 7, 3, "f32", True), (300, 256, 64, 8, "bf16", True), (129, 72, 10, 2, "bf16", False),
+                          (512, 2048, 128, 8, "bf16", True)])
+def test_router_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, dtype, with_scores):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    w = (rng.standard_normal((hidden, experts)) * (0.02 if hidden >= 256 else 0.3)).astype(np.float32)
+    d_weights = rng.standard_normal((tokens, top_k)).astype(np.float32)
+    d_scores = rng.standard_normal((tokens, experts)).astype(np.float32) if with_scores else None
+    scale = 2.5
+    xd, wd = dev(x, gpu, dtype), dev(w, gpu, dtype)
+    fwd = ops.router(xd, wd, None, top_k, scale)
+    cast = lambda a: O.cast_compute(a, dtype)
+    want = G.router_backward(cast(x), cast(w), host(fwd.expert_ids), cast(d_weights), d_scores, scale,
+                             scores=host(fwd.scores))
+    dx, d_w = grad.router_backward(xd, wd, fwd.scores, fwd.expert_ids, dev(d_weights, gpu, dtype),
+                                   None if d_scores is None else dev(d_scores, gpu), scale)
+    tag = f"router grad {dtype} T={tokens} H={hidden} E={experts} K={top_k}"
+    if dtype == "bf16":
+        assert report(tag + " dx", host(dx), want.dx.astype(np.float32)) <= BF16_MAX_REL
+        assert report(tag + " d_w_router", host(d_w), want.d_w_router.astype(np.float32)) <= BF16_MAX_REL
+    else:
+        np.testing.assert_allclose(host(dx), want.dx, rtol=1e-4, atol=2e-5)
+        np.testing.assert_allclose(host(d_w), want.d_w_router, rtol=1e-4, atol=2e-5)
+
+
+def layer_case(gpu, name, tokens, top_k, dtype, tag):
+    inp = O.make_inputs(name, seed=0, tokens=tokens)
+    cfg = inp["cfg"]
+    T = inp["x"].shape[0] * inp["x"].shape[1]
+    x2 = inp["x"].reshape(T, cfg["H"])
+    rng = np.random.default_rng(17)
+    dy = rng.standard_normal(x2.shape).astype(np.float32)
+    d_scores = (rng.standard_normal((T, cfg["E"])) * 0.1).astype(np.float32)
+    params = [dev(inp[k], gpu, dtype) for k in ("w_router", "gate", "up", "down")]
+    shared = None if inp["shared"] is None else tuple(dev(m, gpu, dtype) for m in inp["shared"])
+    xd = dev(x2, gpu, dtype)
+    result, residuals = grad.moe_forward_train(xd, params[0], dev(inp["expert_bias"], gpu), params[1], params[2],
+                                               params[3], top_k, 1.0, shared=shared)
+    plain = ops.moe_forward(xd, params[0], dev(inp["expert_bias"], gpu), params[1], params[2], params[3], top_k, 1.0,
+                            shared=shared)
+    assert torch.equal(plain.expert_ids, result.expert_ids) and torch.equal(plain.y, result.y)
+    got = grad.moe_backward(xd, dev(dy, gpu, dtype), dev(d_scores, gpu), params[0], params[1], params[2], params[3],
+                            shared, result, residuals, 1.0)
+    again = grad.moe_backward(xd, dev(dy, gpu, dtype), dev(d_scores, gpu), params[0], params[1], params[2],
+                              params[3], shared, result, residuals, 1.0)
+    cast = lambda a: O.cast_compute(a, dtype)
+    want = G.moe_backward(cast(x2), cast(inp["w_router"]), cast(inp["gate"]), cast(inp["up"]), cast(inp["down"]),
+                          None if inp["shared"] is None else tuple(cast(m) for m in inp["shared"]),
+                          host(result.expert_ids), host(result.weights), cast(dy), d_scores, 1.0,
+                          scores=host(result.scores))
+    pairs = [("dx", got.dx, want.dx, again.dx), ("d_w_router", got.d_w_router, want.d_w_router, again.d_w_router),
+             ("d_gate", got.d_gate, want.d_gate, again.d_gate), ("d_up", got.d_up, want.d_up, again.d_up),
+             ("d_down", got.d_down, want.d_down, again.d_down)]
+    if shared is not None:
+        for i, n in enumerate(("d_shared_gate", "d_shared_up", "d_shared_down")):
+            pairs.append((n, got.d_shared[i], want.d_shared[i], again.d_shared[i]))
+    for n, g, ref, g2 in pairs:
+        assert torch.equal(g, g2), f"{n} differs between two identical calls"
+        if dtype == "bf16":
+            assert report(f"{tag} {n}", host(g), ref.astype(np.float32)) <= BF16_MAX_REL
+        else:
+            scale = float(np.max(np.abs(ref))) or 1.0
+            np.testing.assert_allclose(host(g) / scale, ref / scale, rtol=1e-4, atol=3e-5, err_msg=n)
+
+
+def test_layer_gradients_c1_fp32_sample(gpu):
+    layer_case(gpu, "C1", 256, 2, "f32", "C1 grad fp32 T=256")
+
+
+def test_layer_gradients_c2_bf16_sample(gpu):
+    layer_case(gpu, "C2", 512, 2, "bf16", "C2 grad bf16 T=512 H=1024 E=16 K=2 I=2816")
+
+
+def test_layer_gradients_c3_bf16_sample_with_shared(gpu):
+    layer_case(gpu, "C3", 512, 8, "bf16", "C3 grad bf16 T=512 H=2048 E=64 K=8 I=1408 Ns=2")
+
+
+def test_gradients_with_no_tokens(gpu):
+    E, H, I, K = 4, 64, 64, 2
+    z = lambda *s: torch.zeros(s, dtype=torch.bfloat16, device=gpu)
+    rnd = lambda *s: torch.randn(s, device=gpu).to(torch.bfloat16)
+    gate, up, down = rnd(E, H, I), rnd(E, H, I), rnd(E, I, H)
+    plan = ops.dispatch(torch.zeros((0, K), dtype=torch.int32, device=gpu), E)
+    res = grad.ExpertResiduals(z(0, I), z(0, I))
+    got = grad.experts_backward(z(0, H), z(0, H), plan, z(0, K), gate, up, down, res)
+    assert got.dx.shape == (0, H) and not got.d_gate.any() and not got.d_up.any() and not got.d_down.any()

@@ -1,0 +1,138 @@
+"""Pins the backward oracle: every analytic gradient against central finite differences of an
+independently written float64 forward (the dense formulation of the reference's own gradient
+test, tests/jaxtitan/test_model.py:596-603), on that test's inputs and routing patterns."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from oracle import moe_grad_oracle as G
+
+
+def silu(z):
+    return z / (1.0 + np.exp(-z))
+
+
+def dense_experts(x, ids, weights, gate, up, down):
+    """reference_output of test_model.py:596-603: gather the selected matrices, three einsums, weighted sum."""
+    sel_gate, sel_up, sel_down = gate[ids], up[ids], down[ids]
+    gate_x = np.einsum("th,tkhi->tki", x, sel_gate)
+    up_x = np.einsum("th,tkhi->tki", x, sel_up)
+    out = np.einsum("tki,tkih->tkh", silu(gate_x) * up_x, sel_down)
+    return np.sum(out * weights[..., None], axis=-2)
+
+
+def numeric_grad(f, a, eps=1e-6):
+    """Central differences of the scalar function f with respect to every element of a."""
+    g = np.zeros_like(a)
+    flat, gf = a.reshape(-1), g.reshape(-1)
+    for i in range(flat.size):
+        keep = flat[i]
+        flat[i] = keep + eps
+        hi = f()
+        flat[i] = keep - eps
+        lo = f()
+        flat[i] = keep
+        gf[i] = (hi - lo) / (2 * eps)
+    return g
+
+
+def reference_case(batch=1):
+    """Inputs of test_model.py:557-588 (flattened over batch and sequence)."""
+    E, H, I, S, K = 4, 3, 4, 6, 2
+    T = batch * S
+    x = np.arange(T * H, dtype=np.float64).reshape(T, H) / 17.0
+    gate = np.arange(E * H * I, dtype=np.float64).reshape(E, H, I) / 37.0
+    up = np.flip(gate, axis=-1) / 1.3
+    down = np.arange(E * I * H, dtype=np.float64).reshape(E, I, H) / 43.0
+    weights = np.tile(np.array([0.3, 0.7]), (T, 1))
+    balanced = (np.arange(T * K).reshape(T, K) % E).astype(np.int32)
+    patterns = {
+        "balanced": balanced,
+        "no_expert_three": balanced % 3,
+        "all_one_expert": np.zeros_like(balanced),
+        "duplicate_routes": np.repeat((np.arange(T) % E).reshape(T, 1), K, axis=-1).astype(np.int32),
+    }
+    cotangent = np.arange(x.size, dtype=np.float64).reshape(x.shape) / float(x.size)
+    return x, gate, up, down, weights, patterns, cotangent
+
+
+@pytest.mark.parametrize("pattern", ["balanced", "no_expert_three", "all_one_expert", "duplicate_routes"])
+@pytest.mark.parametrize("batch", [1, 2])
+def test_experts_backward_matches_finite_differences_on_the_reference_case(pattern, batch):
+    x, gate, up, down, weights, patterns, cot = reference_case(batch)
+    ids = patterns[pattern]
+    got = G.experts_backward(x, ids, weights, gate, up, down, cot)
+    loss = lambda: float(np.sum(dense_experts(x, ids, weights, gate, up, down) * cot))
+    for name, arr, grad in (("x", x, got.dx), ("weights", weights, got.d_weights), ("gate", gate, got.d_gate),
+                            ("up", up, got.d_up), ("down", down, got.d_down)):
+        want = numeric_grad(loss, arr)
+        np.testing.assert_allclose(grad, want, rtol=2e-6, atol=2e-6, err_msg=f"{pattern}: d/d{name}")
+    if pattern == "no_expert_three":
+        assert not got.d_gate[3].any() and not got.d_up[3].any() and not got.d_down[3].any()
+
+
+def test_shared_backward_matches_finite_differences():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((5, 4))
+    gate, up = rng.standard_normal((4, 6)) * 0.5, rng.standard_normal((4, 6)) * 0.5
+    down = rng.standard_normal((6, 4)) * 0.5
+    cot = rng.standard_normal((5, 4))
+    got = G.shared_backward(x, gate, up, down, cot)
+    loss = lambda: float(np.sum(((silu(x @ gate) * (x @ up)) @ down) * cot))
+    for arr, grad in ((x, got.dx), (gate, got.d_gate), (up, got.d_up), (down, got.d_down)):
+        np.testing.assert_allclose(grad, numeric_grad(loss, arr), rtol=2e-6, atol=2e-6)
+
+
+def router_weights_closed_form(x, w, ids, scale):
+    p_all = 1.0 / (1.0 + np.exp(-(x @ w)))
+    p = np.take_along_axis(p_all, ids, axis=-1)
+    return scale * p / (p.sum(-1, keepdims=True) + 1e-20), p_all
+
+
+@pytest.mark.parametrize("with_score_cotangent", [False, True])
+def test_router_backward_matches_finite_differences(with_score_cotangent):
+    rng = np.random.default_rng(4)
+    T, H, E, K, scale = 6, 5, 7, 3, 2.5
+    x, w = rng.standard_normal((T, H)), rng.standard_normal((H, E)) * 0.7
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int64)  # the selection is held fixed
+    d_weights = rng.standard_normal((T, K))
+    d_scores = rng.standard_normal((T, E)) if with_score_cotangent else None
+    got = G.router_backward(x, w, ids, d_weights, d_scores, scale)
+
+    def loss():
+        weights, scores = router_weights_closed_form(x, w, ids, scale)
+        extra = float(np.sum(scores * d_scores)) if with_score_cotangent else 0.0
+        return float(np.sum(weights * d_weights)) + extra
+
+    np.testing.assert_allclose(got.dx, numeric_grad(loss, x), rtol=2e-6, atol=2e-6)
+    np.testing.assert_allclose(got.d_w_router, numeric_grad(loss, w), rtol=2e-6, atol=2e-6)
+
+
+def test_layer_backward_matches_finite_differences():
+    rng = np.random.default_rng(5)
+    T, H, E, K, I, Is, scale = 7, 4, 5, 2, 6, 3, 1.5
+    x, w = rng.standard_normal((T, H)), rng.standard_normal((H, E)) * 0.7
+    gate, up = rng.standard_normal((E, H, I)) * 0.5, rng.standard_normal((E, H, I)) * 0.5
+    down = rng.standard_normal((E, I, H)) * 0.5
+    shared = (rng.standard_normal((H, Is)) * 0.5, rng.standard_normal((H, Is)) * 0.5,
+              rng.standard_normal((Is, H)) * 0.5)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int64)
+    dy, d_scores = rng.standard_normal((T, H)), rng.standard_normal((T, E))
+
+    def layer():
+        weights, scores = router_weights_closed_form(x, w, ids, scale)
+        y = dense_experts(x, ids, weights, gate, up, down) + (silu(x @ shared[0]) * (x @ shared[1])) @ shared[2]
+        return y, scores, weights
+
+    weights0 = layer()[2]
+    got = G.moe_backward(x, w, gate, up, down, shared, ids, weights0, dy, d_scores, scale)
+
+    def loss():
+        y, scores, _ = layer()
+        return float(np.sum(y * dy) + np.sum(scores * d_scores))
+
+    for arr, grad in ((x, got.dx), (w, got.d_w_router), (gate, got.d_gate), (up, got.d_up), (down, got.d_down),
+                      (shared[0], got.d_shared[0]), (shared[1], got.d_shared[1]), (shared[2], got.d_shared[2])):
+        np.testing.assert_allclose(grad, numeric_grad(loss, arr), rtol=5e-6, atol=5e-6)
