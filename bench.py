@@ -98,6 +98,55 @@ def cpu_baseline(name: str, sample_tokens: int) -> dict:
     )
 
 
+def train_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, work) -> dict:
+    """Forward that keeps residuals + backward (all gradients), timed with events over `steps` pairs.
+
+    Not the headline metric (that is the forward layer); reported beside it.  The backward does
+    twice the matrix-product work of the forward: one data-gradient and one weight-gradient
+    product for each forward product.
+    """
+    import torch
+
+    from research_amd import grad
+
+    dev = x.device
+    dy = torch.randn(x.shape, device=dev).to(x.dtype)
+    d_scores = torch.randn((x.shape[0], cfg["E"]), device=dev) * 0.01
+
+    def fwd():
+        return grad.moe_forward_train(x, w_r, bias, gate, upw, down, cfg["K"], 1.0, shared=shared)
+
+    def bwd(result, residuals):
+        return grad.moe_backward(x, dy, d_scores, w_r, gate, upw, down, shared, result, residuals, 1.0)
+
+    result, residuals = fwd()
+    bwd(result, residuals)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    fwd_ms = bwd_ms = 0.0
+    for _ in range(steps):
+        ev[0].record()
+        result, residuals = fwd()
+        ev[1].record()
+        bwd(result, residuals)
+        ev[2].record()
+        ev[2].synchronize()
+        fwd_ms += ev[0].elapsed_time(ev[1])
+        bwd_ms += ev[1].elapsed_time(ev[2])
+    fwd_ms /= steps
+    bwd_ms /= steps
+    gemm_flops = 2.0 * (work["gate_up_flops"] + work["down_flops"] + work["shared_gate_up_flops"]
+                        + work["shared_down_flops"])
+    return {
+        "forward_with_residuals_ms": fwd_ms,
+        "backward_ms": bwd_ms,
+        "tokens_per_s_forward_backward": x.shape[0] / ((fwd_ms + bwd_ms) * 1e-3),
+        "backward_gemm_flops": gemm_flops,
+        "backward_tflops": gemm_flops / (bwd_ms * 1e-3) / 1e12 if bwd_ms > 0 else 0.0,
+        "gradients": "x, router, gate, up, down" + (", shared gate/up/down" if shared is not None else ""),
+    }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -106,6 +155,7 @@ def main() -> int:
     parser.add_argument("--config", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
     parser.add_argument("--cpu-sample-tokens", type=int, default=2048)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-train", action="store_true", help="skip the forward+backward timing")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: the layer runs with every expert local and no collective; "
@@ -291,6 +341,8 @@ def main() -> int:
         "roofline": roofline,
         "stages": stages,
     }
+    if not args.no_train:
+        line["train"] = train_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, work)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.config, min(args.cpu_sample_tokens, T))
     print(json.dumps(line))
