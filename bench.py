@@ -98,8 +98,33 @@ def cpu_baseline(name: str, sample_tokens: int) -> dict:
     )
 
 
+def block_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, layer_ms) -> dict:
+    """x + post_norm(moe(pre_norm(x))): the layer with the decoder block's two RMSNorms and the residual
+    add around it (the post-norm and the add run inside the combine kernel)."""
+    import torch
+
+    from research_amd import ops
+
+    dev = x.device
+    pre = torch.ones((cfg["H"],), dtype=torch.float32, device=dev)
+    post = torch.full((cfg["H"],), 0.5, dtype=torch.float32, device=dev)
+
+    def step():
+        return ops.ffn_block_forward(x, pre, post, 1e-6, w_r, bias, gate, upw, down, cfg["K"], 1.0, shared=shared)
+
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"ms_per_step": ms, "tokens_per_s": x.shape[0] / (ms * 1e-3), "over_layer_ms": ms - layer_ms}
+
+
 def train_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, work) -> dict:
-    """Forward that keeps residuals + backward (all gradients), timed with events over `steps` pairs.
+    """Forward that keeps residuals + backward (all gradients): medians of event timings over `steps` pairs.
 
     Not the headline metric (that is the forward layer); reported beside it.  The backward does
     twice the matrix-product work of the forward: one data-gradient and one weight-gradient
@@ -119,11 +144,12 @@ def train_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, work) -> dic
     def bwd(result, residuals):
         return grad.moe_backward(x, dy, d_scores, w_r, gate, upw, down, shared, result, residuals, 1.0)
 
-    result, residuals = fwd()
-    bwd(result, residuals)
+    for _ in range(3):  # lets torch's caching allocator settle on the buffers it will reuse
+        result, residuals = fwd()
+        bwd(result, residuals)
     torch.cuda.synchronize()
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
-    fwd_ms = bwd_ms = 0.0
+    fwd_all, bwd_all = [], []
     for _ in range(steps):
         ev[0].record()
         result, residuals = fwd()
@@ -131,10 +157,10 @@ def train_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, work) -> dic
         bwd(result, residuals)
         ev[2].record()
         ev[2].synchronize()
-        fwd_ms += ev[0].elapsed_time(ev[1])
-        bwd_ms += ev[1].elapsed_time(ev[2])
-    fwd_ms /= steps
-    bwd_ms /= steps
+        fwd_all.append(ev[0].elapsed_time(ev[1]))
+        bwd_all.append(ev[1].elapsed_time(ev[2]))
+    fwd_ms = statistics.median(fwd_all)
+    bwd_ms = statistics.median(bwd_all)
     gemm_flops = 2.0 * (work["gate_up_flops"] + work["down_flops"] + work["shared_gate_up_flops"]
                         + work["shared_down_flops"])
     return {
@@ -341,6 +367,7 @@ def main() -> int:
         "roofline": roofline,
         "stages": stages,
     }
+    line["block"] = block_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, ms_per_step)
     if not args.no_train:
         line["train"] = train_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, work)
     if not args.no_cpu_baseline:

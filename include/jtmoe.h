@@ -222,6 +222,48 @@ int jtmoe_moe_forward_timed(const void* x, const void* w_router, const float* ex
                             float* stage_ms);
 
 /* ------------------------------------------------------------------------------------------
+ * The decoder block around the layer (blocks.py:224-230):
+ *     x = x + ffn_post_norm(mlp(ffn_pre_norm(x)))
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * RMSNorm over the last axis.  Replaces the modules of build_rms_norm
+ * (models/components/norm.py:12-31: flax nnx.RMSNorm, float32 scale) and the reference's
+ * forward-only kernel boundary rmsnorm_reference / rmsnorm_tk_forward
+ * (kernels/rmsnorm.py:14-52, kernels/cuda/rmsnorm/rmsnorm_ffi.cu):
+ *   y = round_dtype( f32(x) * (1/sqrt(mean(f32(x)^2) + eps) * scale) ),  scale float32 [H].
+ */
+int jtmoe_rmsnorm(const void* x, const float* scale, int64_t T, int64_t H, double eps, int dtype,
+                  void* y, void* stream);
+
+/*
+ * jtmoe_combine followed, inside the same kernel, by the block's tail:
+ *   out[t] = round( residual[t] + rmsnorm(y[t]; post_scale, eps) ),  y = the plain combine result.
+ */
+int jtmoe_combine_norm_residual(const void* packed_y, const int32_t* inverse, const void* weights,
+                                const void* shared_y, const void* residual, const float* post_scale,
+                                double eps, int64_t T, int64_t H, int64_t K, int dtype,
+                                void* out, void* stream);
+
+/*
+ * The block's second half in one call: out = x + rmsnorm(moe(rmsnorm(x; pre_scale)); post_scale).
+ * Router outputs and dispatch plan as in jtmoe_moe_forward (they refer to the normalised x).
+ */
+size_t jtmoe_ffn_block_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                                       int dtype);
+int jtmoe_ffn_block_forward(const void* x, const float* pre_scale, const float* post_scale, double eps,
+                            const void* w_router, const float* expert_bias,
+                            const void* gate, const void* up, const void* down,
+                            const void* shared_gate, const void* shared_up, const void* shared_down,
+                            int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                            double route_scale, int dtype,
+                            void* out, int32_t* expert_ids, void* weights, float* scores,
+                            float* expert_counts, float* importance,
+                            int32_t* group_sizes, int32_t* offsets,
+                            int32_t* source_order, int32_t* inverse,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Training: forward passes that keep residuals, and the vector-Jacobian products.
  *
  * The reference trains SparseMoE through JAX automatic differentiation and requires a

@@ -14,6 +14,7 @@ in NumPy, the algorithm of the reference layer
 * ``router_stats``      <- ``_router_stats``                     moe.py:794-825
 * ``sequence_balance_loss`` <- ``_sequence_balance_loss``        moe.py:828-840
 * ``moe_forward``       <- ``SparseMoE.forward_with_output``     moe.py:418-446
+* ``rmsnorm`` / ``ffn_block_forward`` <- the block around the layer  blocks.py:224-230, norm.py:12-31
 
 The arithmetic the reference delegates to jax 0.10.0 / jaxlib 0.10.0 (pinned
 in the reference's ``uv.lock``; absent from this environment) is restated from
@@ -49,6 +50,10 @@ Parity status of each function (what pins it is exercised in
 * shared_swiglu: pinned by test_model.py:873-884 (zeroed routed experts).
 * router_stats / sequence_balance_loss: pinned by test_model.py:242-252 and
   :905-908 and closed forms.
+* rmsnorm: pinned by the reference's known-answer test (tests/jaxtitan/test_kernels.py:192-204),
+  a float64 closed form and the scale-invariance property rmsnorm(c x) = rmsnorm(x) at eps = 0.
+  Which of two equally valid fp32 multiplication orders flax uses: PARITY UNPINNED at the
+  last-ulp level (flax is absent; nothing in the reference's tests distinguishes them).
 
 The scores use a fully specified fp32 sigmoid (``sigmoid_f32``) built only
 from IEEE-754 add, multiply, divide, round-to-integer and power-of-two scaling,
@@ -466,6 +471,40 @@ def moe_forward(
             top_k,
         )
     return MoeResult(y.reshape(batch, seq_len, hidden), route, disp, packed_y, stats, aux)
+
+
+# --------------------------------------------------------------------------
+# the decoder block around the layer: x + post_norm(mlp(pre_norm(x)))
+# --------------------------------------------------------------------------
+def rmsnorm(x: np.ndarray, scale: np.ndarray, eps: float, dtype: str) -> np.ndarray:
+    """RMSNorm over the last axis with a float32 scale.
+
+    The modules are flax ``nnx.RMSNorm`` (models/components/norm.py:12-31; flax 0.12.7 in
+    the reference's ``uv.lock``, absent here), whose published algorithm is: statistics in
+    float32, ``mul = rsqrt(mean(x^2) + eps) * scale``, ``y = x * mul``, cast to the compute
+    dtype.  The reference's own ``rmsnorm_reference`` (kernels/rmsnorm.py:14-21) multiplies in
+    the order ``(x * inv_rms) * weight``; both orders round to the same bf16 value except for
+    results that sit within one fp32 ulp of a bf16 rounding boundary.  The sum of squares is
+    accumulated by ``numpy.sum`` (pairwise), not in the order of any particular kernel.
+    """
+    xc = cast_compute(x, dtype).astype(np.float32)
+    var = np.sum(xc * xc, axis=-1, keepdims=True, dtype=np.float32) / np.float32(xc.shape[-1])
+    inv = np.float32(1.0) / np.sqrt(var + np.float32(eps), dtype=np.float32)
+    mul = inv * np.asarray(scale, dtype=np.float32)
+    return cast_compute(xc * mul, dtype)
+
+
+def ffn_block_forward(x, pre_scale, post_scale, eps, w_router, expert_bias, gate, up, down, top_k,
+                      route_scale=1.0, dtype="f32", shared=None):
+    """x + ffn_post_norm(mlp(ffn_pre_norm(x))) of the decoder block (blocks.py:224-230); x [B,S,H].
+
+    Returns (out [B,S,H], MoeResult of the inner layer).
+    """
+    xc = cast_compute(np.asarray(x, dtype=np.float32), dtype)
+    normed = rmsnorm(xc, pre_scale, eps, dtype)
+    inner = moe_forward(normed, w_router, expert_bias, gate, up, down, top_k, route_scale, dtype, shared)
+    out = cast_compute(xc + rmsnorm(inner.y, post_scale, eps, dtype), dtype)
+    return out, inner
 
 
 # --------------------------------------------------------------------------

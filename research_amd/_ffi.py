@@ -59,6 +59,16 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_ptr] * 9 + [c_i64] * 6 + [c_dbl, c_int] + [c_ptr] * 10 + [c_ptr, c_size, c_ptr],
     ),
+    "jtmoe_rmsnorm": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_dbl, c_int, c_ptr, c_ptr]),
+    "jtmoe_combine_norm_residual": (
+        c_int,
+        [c_ptr] * 6 + [c_dbl] + [c_i64] * 3 + [c_int, c_ptr, c_ptr],
+    ),
+    "jtmoe_ffn_block_workspace_bytes": (c_size, [c_i64] * 6 + [c_int]),
+    "jtmoe_ffn_block_forward": (
+        c_int,
+        [c_ptr] * 3 + [c_dbl] + [c_ptr] * 8 + [c_i64] * 6 + [c_dbl, c_int] + [c_ptr] * 10 + [c_ptr, c_size, c_ptr],
+    ),
     "jtmoe_grouped_swiglu_train": (
         c_int,
         [c_ptr] * 7 + [c_i64] * 5 + [c_int] + [c_ptr] * 5,

@@ -254,7 +254,8 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
                             float* scores, float* expert_counts, float* importance, int32_t* group_sizes,
                             int32_t* offsets, int32_t* source_order, int32_t* inverse, void* workspace,
                             size_t workspace_bytes, void* stream, void* gate_pre, void* up_pre,
-                            void* shared_gate_pre, void* shared_up_pre) {
+                            void* shared_gate_pre, void* shared_up_pre, const void* residual = nullptr,
+                            const float* post_scale = nullptr, double eps = 0.0) {
   clear_error();
   const bool train = gate_pre != nullptr;
   JT_REQUIRE(dtype_ok(dtype), "moe_forward: unknown dtype %d", dtype);
@@ -298,7 +299,11 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
                                stream);
     if (rc) return rc;
   }
-  rc = jtmoe_combine(w.packed_y, inverse, weights, Is > 0 ? w.shared_y : nullptr, T, H, K, dtype, y, stream);
+  if (residual)  // the decoder block's tail fused into the combine: y = residual + rmsnorm(layer output)
+    rc = jtmoe_combine_norm_residual(w.packed_y, inverse, weights, Is > 0 ? w.shared_y : nullptr, residual, post_scale,
+                                     eps, T, H, K, dtype, y, stream);
+  else
+    rc = jtmoe_combine(w.packed_y, inverse, weights, Is > 0 ? w.shared_y : nullptr, T, H, K, dtype, y, stream);
   stage_mark(kStageCombine, as_stream(stream));
   return rc;
 }
@@ -329,12 +334,46 @@ extern "C" int jtmoe_moe_forward_train(const void* x, const void* w_router, cons
     clear_error();
     return fail(JTMOE_EINVAL, "moe_forward_train: null residual buffer");
   }
-  // the address of a local stands in for the residual pointers when there are no tokens
-  int none = 0;
+  // without tokens there is nothing to keep and the plain path (which launches nothing) serves
   return moe_forward_impl(x, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H, E, K, I,
                           Is, route_scale, dtype, y, expert_ids, weights, scores, expert_counts, importance,
                           group_sizes, offsets, source_order, inverse, workspace, workspace_bytes, stream,
-                          gate_pre ? gate_pre : &none, up_pre ? up_pre : &none, shared_gate_pre, shared_up_pre);
+                          gate_pre, up_pre, shared_gate_pre, shared_up_pre);
+}
+
+extern "C" size_t jtmoe_ffn_block_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                                                  int dtype) {
+  const size_t layer = jtmoe_workspace_bytes(T, H, E, K, I, Is, dtype);
+  if (layer == 0) return 0;
+  return layer + align_up((size_t)T * (size_t)H * dtype_bytes(dtype), 256);
+}
+
+extern "C" int jtmoe_ffn_block_forward(const void* x, const float* pre_scale, const float* post_scale, double eps,
+                                       const void* w_router, const float* expert_bias, const void* gate,
+                                       const void* up, const void* down, const void* shared_gate,
+                                       const void* shared_up, const void* shared_down, int64_t T, int64_t H,
+                                       int64_t E, int64_t K, int64_t I, int64_t Is, double route_scale, int dtype,
+                                       void* out, int32_t* expert_ids, void* weights, float* scores,
+                                       float* expert_counts, float* importance, int32_t* group_sizes,
+                                       int32_t* offsets, int32_t* source_order, int32_t* inverse, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  clear_error();
+  JT_REQUIRE(dtype_ok(dtype), "ffn_block_forward: unknown dtype %d", dtype);
+  JT_REQUIRE(T >= 0 && H > 0 && E > 0 && K > 0 && I > 0 && Is >= 0, "ffn_block_forward: shape out of range");
+  JT_REQUIRE(pre_scale && post_scale, "ffn_block_forward: null norm scale");
+  JT_REQUIRE(workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
+             "ffn_block_forward: workspace must be non-null and 256-byte aligned");
+  const size_t layer_bytes = jtmoe_workspace_bytes(T, H, E, K, I, Is, dtype);
+  const size_t need = jtmoe_ffn_block_workspace_bytes(T, H, E, K, I, Is, dtype);
+  if (workspace_bytes < need)
+    return fail(JTMOE_EWORKSPACE, "ffn_block_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+  void* normed = static_cast<unsigned char*>(workspace) + layer_bytes;
+  int rc = jtmoe_rmsnorm(x, pre_scale, T, H, eps, dtype, normed, stream);
+  if (rc) return rc;
+  return moe_forward_impl(normed, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H, E,
+                          K, I, Is, route_scale, dtype, out, expert_ids, weights, scores, expert_counts, importance,
+                          group_sizes, offsets, source_order, inverse, workspace, layer_bytes, stream, nullptr,
+                          nullptr, nullptr, nullptr, T > 0 ? x : nullptr, post_scale, eps);
 }
 
 extern "C" int jtmoe_moe_forward_timed(const void* x, const void* w_router, const float* expert_bias,

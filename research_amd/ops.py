@@ -324,6 +324,56 @@ def combine(
     return y
 
 
+def rmsnorm(x: torch.Tensor, scale: torch.Tensor, eps: float = 1.0e-6) -> torch.Tensor:
+    """RMSNorm over the last axis of x [..., H] with a float32 scale [H]."""
+    _check(x, "x")
+    if x.dim() < 2:
+        raise ContractError("rmsnorm input rank must be at least 2")
+    hidden = x.shape[-1]
+    _check(scale, "scale", torch.float32, (hidden,))
+    if eps < 0:
+        raise ContractError("eps must not be negative")
+    rows = x.numel() // hidden
+    y = torch.empty_like(x)
+    status = _lib().jtmoe_rmsnorm(_ptr(x), _ptr(scale), rows, hidden, float(eps), _code(x.dtype), _ptr(y),
+                                  _stream(x.device))
+    _raise(status, "jtmoe_rmsnorm")
+    return y
+
+
+def combine_norm_residual(
+    packed_y: torch.Tensor,
+    inverse: torch.Tensor,
+    weights: torch.Tensor,
+    residual: torch.Tensor,
+    post_scale: torch.Tensor,
+    eps: float = 1.0e-6,
+    shared_y: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """residual + rmsnorm(combine(packed_y, inverse, weights, shared_y); post_scale) in one kernel."""
+    _check(packed_y, "packed_y")
+    _check(weights, "weights", packed_y.dtype)
+    if packed_y.dim() != 2 or weights.dim() != 2:
+        raise ContractError("combine expects packed_y [rows, hidden] and weights [tokens, top_k]")
+    tokens, top_k = weights.shape
+    rows, hidden = packed_y.shape
+    if rows != tokens * top_k:
+        raise ContractError(f"packed_y has {rows} rows, expected tokens*top_k = {tokens * top_k}")
+    _check(inverse, "inverse", torch.int32, (rows,))
+    _check(residual, "residual", packed_y.dtype, (tokens, hidden))
+    _check(post_scale, "post_scale", torch.float32, (hidden,))
+    if shared_y is not None:
+        _check(shared_y, "shared_y", packed_y.dtype, (tokens, hidden))
+    dev = packed_y.device
+    out = torch.empty((tokens, hidden), dtype=packed_y.dtype, device=dev)
+    status = _lib().jtmoe_combine_norm_residual(
+        _ptr(packed_y), _ptr(inverse), _ptr(weights), _ptr(shared_y), _ptr(residual), _ptr(post_scale), float(eps),
+        tokens, hidden, top_k, _code(packed_y.dtype), _ptr(out), _stream(dev),
+    )
+    _raise(status, "jtmoe_combine_norm_residual")
+    return out
+
+
 def router_stats(expert_counts: torch.Tensor) -> torch.Tensor:
     """expert_counts [E] f32 -> [6] f32: total, min, max, mean, max_vio, entropy."""
     _check(expert_counts, "expert_counts", torch.float32)
@@ -470,4 +520,77 @@ def moe_forward(
         stage_ms[:] = list(buf)
     _raise(status, "jtmoe_moe_forward")
     return LayerResult(y, expert_ids, weights, scores, expert_counts, importance,
+                       group_sizes, offsets, source_order, inverse)
+
+
+def ffn_block_forward(
+    x: torch.Tensor,
+    pre_scale: torch.Tensor,
+    post_scale: torch.Tensor,
+    eps: float,
+    w_router: torch.Tensor,
+    expert_bias: torch.Tensor | None,
+    gate: torch.Tensor,
+    up: torch.Tensor,
+    down: torch.Tensor,
+    top_k: int,
+    route_scale: float = 1.0,
+    shared: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
+) -> LayerResult:
+    """x + post_norm(moe(pre_norm(x))) on x [T,H] through jtmoe_ffn_block_forward; ``y`` of the result is the block output."""
+    _check(x, "x")
+    if x.dim() != 2:
+        raise ContractError(f"x must have shape [tokens, hidden], got {list(x.shape)}")
+    tokens, hidden = x.shape
+    _check(pre_scale, "pre_scale", torch.float32, (hidden,))
+    _check(post_scale, "post_scale", torch.float32, (hidden,))
+    _check(w_router, "w_router", x.dtype)
+    if w_router.dim() != 2 or w_router.shape[0] != hidden:
+        raise ContractError(f"w_router must have shape [{hidden}, experts], got {list(w_router.shape)}")
+    experts = w_router.shape[1]
+    _validate_router_attrs(experts, top_k, route_scale)
+    if expert_bias is not None:
+        _check(expert_bias, "expert_bias", torch.float32, (experts,))
+    _check(gate, "gate", x.dtype)
+    if gate.dim() != 3 or gate.shape[0] != experts or gate.shape[1] != hidden:
+        raise ContractError(f"expert gate must have shape [{experts}, {hidden}, inter], got {list(gate.shape)}")
+    inter = gate.shape[2]
+    _check(up, "up", x.dtype, (experts, hidden, inter))
+    _check(down, "down", x.dtype, (experts, inter, hidden))
+    shared_inter = 0
+    sg = su = sd = None
+    if shared is not None:
+        sg, su, sd = shared
+        _check(sg, "shared gate", x.dtype)
+        if sg.dim() != 2 or sg.shape[0] != hidden:
+            raise ContractError(f"shared gate must have shape [{hidden}, inter], got {list(sg.shape)}")
+        shared_inter = sg.shape[1]
+        _check(su, "shared up", x.dtype, (hidden, shared_inter))
+        _check(sd, "shared down", x.dtype, (shared_inter, hidden))
+    dev = x.device
+    n_assign = tokens * top_k
+    i32, f32 = torch.int32, torch.float32
+    out = torch.empty_like(x)
+    expert_ids = torch.empty((tokens, top_k), dtype=i32, device=dev)
+    weights = torch.empty((tokens, top_k), dtype=x.dtype, device=dev)
+    scores = torch.empty((tokens, experts), dtype=f32, device=dev)
+    expert_counts = torch.empty((experts,), dtype=f32, device=dev)
+    importance = torch.empty((experts,), dtype=f32, device=dev)
+    group_sizes = torch.empty((experts,), dtype=i32, device=dev)
+    offsets = torch.empty((experts,), dtype=i32, device=dev)
+    source_order = torch.empty((n_assign,), dtype=i32, device=dev)
+    inverse = torch.empty((n_assign,), dtype=i32, device=dev)
+    lib = _lib()
+    nbytes = lib.jtmoe_ffn_block_workspace_bytes(tokens, hidden, experts, top_k, inter, shared_inter, _code(x.dtype))
+    workspace = layer_workspace(nbytes, dev)
+    status = lib.jtmoe_ffn_block_forward(
+        _ptr(x), _ptr(pre_scale), _ptr(post_scale), float(eps), _ptr(w_router), _ptr(expert_bias),
+        _ptr(gate), _ptr(up), _ptr(down), _ptr(sg), _ptr(su), _ptr(sd),
+        tokens, hidden, experts, top_k, inter, shared_inter, float(route_scale), _code(x.dtype),
+        _ptr(out), _ptr(expert_ids), _ptr(weights), _ptr(scores), _ptr(expert_counts), _ptr(importance),
+        _ptr(group_sizes), _ptr(offsets), _ptr(source_order), _ptr(inverse),
+        workspace.data_ptr(), workspace.numel(), _stream(dev),
+    )
+    _raise(status, "jtmoe_ffn_block_forward")
+    return LayerResult(out, expert_ids, weights, scores, expert_counts, importance,
                        group_sizes, offsets, source_order, inverse)
