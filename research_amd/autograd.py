@@ -1,0 +1,50 @@
+"""The layer as a differentiable torch operation: forward through jtmoe_moe_forward_train, backward
+through jtmoe_moe_backward.
+
+This is the torch-side analogue of the custom VJP the reference asks of a forward-only kernel before
+it may replace a training component (docs/kernel_backend_design.md:120-128): the forward keeps the
+residuals, the backward consumes the cotangents of the two differentiable outputs (the layer output
+and the router scores, which the sequence-balance loss reads, moe.py:828-840).  The expert bias
+only enters the selection and receives no gradient (moe.py:139-140).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from research_amd import grad
+
+
+class MoeLayerFunction(torch.autograd.Function):
+    """(x, w_router, gate, up, down, shared_gate, shared_up, shared_down) -> (y, scores, expert_ids)."""
+
+    @staticmethod
+    def forward(ctx, x, w_router, gate, up, down, shared_gate, shared_up, shared_down, expert_bias, top_k,
+                route_scale):
+        shared = None if shared_gate is None else (shared_gate, shared_up, shared_down)
+        result, residuals = grad.moe_forward_train(x, w_router, expert_bias, gate, up, down, top_k, route_scale,
+                                                   shared=shared)
+        ctx.result, ctx.residuals = result, residuals
+        ctx.route_scale = route_scale
+        ctx.has_shared = shared is not None
+        ctx.save_for_backward(x, w_router, gate, up, down, *(shared or ()))
+        ctx.mark_non_differentiable(result.expert_ids)
+        return result.y, result.scores, result.expert_ids
+
+    @staticmethod
+    def backward(ctx, dy, d_scores, _d_ids):
+        saved = ctx.saved_tensors
+        x, w_router, gate, up, down = saved[:5]
+        shared = tuple(saved[5:8]) if ctx.has_shared else None
+        if dy is None:
+            dy = torch.zeros_like(x)
+        g = grad.moe_backward(x, dy.contiguous(), None if d_scores is None else d_scores.contiguous(), w_router, gate,
+                              up, down, shared, ctx.result, ctx.residuals, ctx.route_scale)
+        ds = g.d_shared if g.d_shared is not None else (None, None, None)
+        return g.dx, g.d_w_router, g.d_gate, g.d_up, g.d_down, ds[0], ds[1], ds[2], None, None, None
+
+
+def moe_layer(x, w_router, expert_bias, gate, up, down, top_k, route_scale=1.0, shared=None):
+    """Differentiable layer on x [T,H]: returns (y [T,H], scores [T,E] float32, expert_ids [T,K] int32)."""
+    sg, su, sd = shared if shared is not None else (None, None, None)
+    return MoeLayerFunction.apply(x, w_router, gate, up, down, sg, su, sd, expert_bias, top_k, float(route_scale))

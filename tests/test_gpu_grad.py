@@ -200,3 +200,29 @@ def test_gradients_with_no_tokens(gpu):
     res = grad.ExpertResiduals(z(0, I), z(0, I))
     got = grad.experts_backward(z(0, H), z(0, H), plan, z(0, K), gate, up, down, res)
     assert got.dx.shape == (0, H) and not got.d_gate.any() and not got.d_up.any() and not got.d_down.any()
+
+
+def test_autograd_function_routes_cotangents_to_the_backward_entry(gpu):
+    """torch.autograd over the layer gives what jtmoe_moe_backward gives for the same cotangents."""
+    from research_amd import autograd
+
+    inp = O.make_inputs("C2", seed=2, tokens=256)
+    cfg = inp["cfg"]
+    x2 = inp["x"].reshape(-1, cfg["H"])
+    leaf = lambda a: dev(a, gpu, "bf16").requires_grad_(True)
+    x, w, gate, up, down = (leaf(a) for a in (x2, inp["w_router"], inp["gate"], inp["up"], inp["down"]))
+    bias = dev(inp["expert_bias"], gpu)
+    y, scores, ids = autograd.moe_layer(x, w, bias, gate, up, down, 2, 1.0)
+    assert not ids.requires_grad and y.requires_grad and scores.requires_grad
+    rng = np.random.default_rng(23)
+    dy = dev(rng.standard_normal(x2.shape).astype(np.float32), gpu, "bf16")
+    d_scores = dev((rng.standard_normal(scores.shape) * 0.1).astype(np.float32), gpu)
+    loss = (y.float() * dy.float()).sum() + (scores * d_scores).sum()
+    loss.backward()
+    result, residuals = grad.moe_forward_train(x.detach(), w.detach(), bias, gate.detach(), up.detach(),
+                                               down.detach(), 2, 1.0)
+    want = grad.moe_backward(x.detach(), dy, d_scores, w.detach(), gate.detach(), up.detach(), down.detach(), None,
+                             result, residuals, 1.0)
+    for got, ref in ((x.grad, want.dx), (w.grad, want.d_w_router), (gate.grad, want.d_gate), (up.grad, want.d_up),
+                     (down.grad, want.d_down)):
+        assert torch.equal(got, ref)
