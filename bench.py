@@ -98,6 +98,25 @@ def cpu_baseline(name: str, sample_tokens: int) -> dict:
     )
 
 
+def graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps) -> dict:
+    """Small batches are bound by launching the layer's kernels from Python, not by the kernels: the same
+    calls captured once into a HIP graph and replayed."""
+    import torch
+
+    from research_amd.graph import GraphedLayer
+
+    layer = GraphedLayer(x, w_r, bias, gate, upw, down, cfg["K"], 1.0, shared=shared)
+    for _ in range(3):
+        layer.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        layer.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"ms_per_step": ms, "tokens_per_s": x.shape[0] / (ms * 1e-3), "steps": steps}
+
+
 def block_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, layer_ms) -> dict:
     """x + post_norm(moe(pre_norm(x))): the layer with the decoder block's two RMSNorms and the residual
     add around it (the post-norm and the add run inside the combine kernel)."""
@@ -148,19 +167,18 @@ def train_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, work) -> dic
         result, residuals = fwd()
         bwd(result, residuals)
     torch.cuda.synchronize()
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
-    fwd_all, bwd_all = [], []
-    for _ in range(steps):
-        ev[0].record()
+    # events are recorded for every step and read after one final synchronisation, so that the host
+    # runs ahead of the GPU as it does in a training loop (no idle gaps from launch latency)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for e in ev:
+        e[0].record()
         result, residuals = fwd()
-        ev[1].record()
+        e[1].record()
         bwd(result, residuals)
-        ev[2].record()
-        ev[2].synchronize()
-        fwd_all.append(ev[0].elapsed_time(ev[1]))
-        bwd_all.append(ev[1].elapsed_time(ev[2]))
-    fwd_ms = statistics.median(fwd_all)
-    bwd_ms = statistics.median(bwd_all)
+        e[2].record()
+    torch.cuda.synchronize()
+    fwd_ms = statistics.median(e[0].elapsed_time(e[1]) for e in ev)
+    bwd_ms = statistics.median(e[1].elapsed_time(e[2]) for e in ev)
     gemm_flops = 2.0 * (work["gate_up_flops"] + work["down_flops"] + work["shared_gate_up_flops"]
                         + work["shared_down_flops"])
     return {
@@ -367,6 +385,8 @@ def main() -> int:
         "roofline": roofline,
         "stages": stages,
     }
+    if T <= 2048:
+        line["graph_replay"] = graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, max(args.steps, 50))
     line["block"] = block_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, ms_per_step)
     if not args.no_train:
         line["train"] = train_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, work)

@@ -346,6 +346,23 @@ static void time_launches(const char* name, double flops, int iters, F launch_on
 // rows that are 16384 token rows fetched through a permutation, hidden 2048, intermediate 1408
 static void time_backward() {
   const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
+  {  // forward gate/up launch that also stores the two products for the backward pass
+    Problem p = make(E, rows, H, I, 20, false, topk, 1.0f);
+    uint16_t *s0, *s1;
+    CK(hipMalloc(&s0, (size_t)rows * I * 2)); CK(hipMalloc(&s1, (size_t)rows * I * 2));
+    auto kernel = grouped_gemm_dma_kernel<GateUpCfg>;
+    CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                           (int)GateUpCfg::SMEM_BYTES));
+    const long mt = (rows + GateUpCfg::BM - 1) / GateUpCfg::BM + E, nt = (I + GateUpCfg::BN - 1) / GateUpCfg::BN;
+    for (int save = 0; save < 2; ++save)
+      time_launches(save ? "forward gate/up, products kept" : "forward gate/up", 4.0 * rows * H * I, 10, [&] {
+        kernel<<<(unsigned)gemm_grid(mt, nt), GateUpCfg::NT, GateUpCfg::SMEM_BYTES>>>(
+            p.A, p.B0, p.B1, p.C, p.dgs, p.doff, E, rows, H, I, (int)mt, (int)nt, p.dmap, topk, p.a_rows,
+            save ? s0 : nullptr, save ? s1 : nullptr);
+      });
+    hipFree(s0); hipFree(s1);
+    release(p);
+  }
   {  // d act = dy[token of row] @ Wd^T : A gathered [T, H], B [E, I, H]
     Problem p = make(E, rows, H, I, 21, false, topk, 1.0f);
     time_launches("dgrad down (gathered dy @ Wd^T)", 2.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(p, nullptr, 1, false); });

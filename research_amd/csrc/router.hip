@@ -289,67 +289,106 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(w), 0, H * E * 2, kBufferFlags);
 
-  u32x4_t a_cur[2], a_nxt[2], w_reg[CW];
+  // Loads run D chunks ahead of the MFMAs through a ring of registers (chunk c lives in slot
+  // c % D), so that the latency of a load is hidden by D - 1 whole iterations instead of by the
+  // few MFMAs of one: with a single chunk in flight every iteration waits for memory.
+  constexpr int D = CW <= 8 ? 3 : (CW <= 16 ? 2 : 1);
+  constexpr int UNROLL = D == 3 ? 6 : 2;  // a multiple of D and of the two LDS stages
+  u32x4_t a_ring[D][2], w_ring[D][CW];
   f32x4_t acc[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[nb][i] = 0.0f;
 
-#define JT_LOAD_W(k0)                                                                        \
+#define JT_LOAD_W(slot, k0)                                                                  \
   _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                           \
     const int c = tid + i * kRouterThreads;                                                  \
     if (W_CHUNKS % kRouterThreads == 0 || c < W_CHUNKS)                                      \
-      w_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c * 16, (k0)*E * 2, 0);       \
+      w_ring[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c * 16, (k0)*E * 2, 0); \
   }
-#define JT_STORE_W(stage)                                                                    \
+#define JT_STORE_W(slot, stage)                                                              \
   _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                           \
     const int c = tid + i * kRouterThreads;                                                  \
     if (W_CHUNKS % kRouterThreads == 0 || c < W_CHUNKS) {                                    \
       const int kr = c / CPR, nc = c - kr * CPR;                                             \
-      *reinterpret_cast<u32x4_t*>(Ws + ((stage)*kRouterKC + kr) * WS + nc * 8) = w_reg[i];   \
+      *reinterpret_cast<u32x4_t*>(Ws + ((stage)*kRouterKC + kr) * WS + nc * 8) = w_ring[slot][i]; \
     }                                                                                        \
   }
-#define JT_LOAD_X(dst, k0)                                                                   \
+#define JT_LOAD_X(slot, k0)                                                                  \
   {                                                                                          \
-    dst[0] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff, (k0)*2, 0);               \
-    dst[1] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff + 16, (k0)*2, 0);          \
+    a_ring[slot][0] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff, (k0)*2, 0);      \
+    a_ring[slot][1] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff + 16, (k0)*2, 0); \
   }
 
   // transposing read of this lane: 16-lane group kg = lane/16 reads rows kg*16 + 8*s + 4*h + i/4
   const int w_lane = ((lane >> 4) * 16 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
   const int nchunks = H / kRouterKC;
-  JT_LOAD_W(0);
-  JT_LOAD_X(a_cur, 0);
-  JT_STORE_W(0);
-  __syncthreads();
-  for (int kc = 0; kc < nchunks; ++kc) {
-    const int stage = kc & 1;
-    if (kc + 1 < nchunks) {
-      JT_LOAD_W((kc + 1) * kRouterKC);
-      JT_LOAD_X(a_nxt, (kc + 1) * kRouterKC);
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nchunks) {
+      JT_LOAD_W(d, d * kRouterKC);
+      JT_LOAD_X(d, d * kRouterKC);
     }
-    const uint16_t* wbase = Ws + stage * kRouterKC * WS + w_lane;
+  JT_STORE_W(0, 0);
+  __syncthreads();
+  for (int kc0 = 0; kc0 < nchunks; kc0 += UNROLL) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_cur[s]);
+    for (int j = 0; j < UNROLL; ++j) {
+      const int kc = kc0 + j;
+      if (kc < nchunks) {  // uniform over the workgroup
+        constexpr int kStages = 2;
+        const int stage = j % kStages, slot = j % D, next_slot = (j + 1) % D;
+        if (D == 1 && kc + 1 < nchunks) {
+          // one slot: it is refilled before the MFMAs, which copy the operand out first
+          const u32x4_t a0 = a_ring[0][0], a1 = a_ring[0][1];
+          JT_LOAD_W(0, (kc + 1) * kRouterKC);
+          JT_LOAD_X(0, (kc + 1) * kRouterKC);
+          const uint16_t* wbase = Ws + stage * kRouterKC * WS + w_lane;
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        const uint16_t* p = wbase + s * 8 * WS + nb * 16;
-        const s16x4_t lo =
-            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
-        const s16x4_t hi =
-            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
-        const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
+          for (int s = 0; s < 2; ++s) {
+            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, s ? a1 : a0);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              const uint16_t* p = wbase + s * 8 * WS + nb * 16;
+              const s16x4_t lo =
+                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+              const s16x4_t hi =
+                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
+              const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+              acc[nb] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
+            }
+          }
+          JT_STORE_W(0, stage ^ 1);
+        } else {
+          const uint16_t* wbase = Ws + stage * kRouterKC * WS + w_lane;
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_ring[slot][s]);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              const uint16_t* p = wbase + s * 8 * WS + nb * 16;
+              const s16x4_t lo =
+                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+              const s16x4_t hi =
+                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
+              const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+              acc[nb] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
+            }
+          }
+          if (D > 1) {
+            if (kc + 1 < nchunks) JT_STORE_W(next_slot, stage ^ 1);
+            if (kc + D < nchunks) {
+              JT_LOAD_W(slot, (kc + D) * kRouterKC);
+              JT_LOAD_X(slot, (kc + D) * kRouterKC);
+            }
+          }
+        }
+        __syncthreads();
       }
     }
-    if (kc + 1 < nchunks) {
-      JT_STORE_W(stage ^ 1);
-      a_cur[0] = a_nxt[0];
-      a_cur[1] = a_nxt[1];
-    }
-    __syncthreads();
   }
 #undef JT_LOAD_W
 #undef JT_STORE_W
@@ -386,9 +425,9 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
   const bool mfma = Elem<T>::is_bf16 && !kFromLogits && H % kRouterKC == 0 && H * E < ((int64_t)1 << 30) &&
                     (E == 16 || E == 32 || E == 64 || E == 128 || E == 256) && aligned16(x) && aligned16(w);
   if (mfma) {
-    // two waves (32 tokens) per workgroup: several workgroups share a CU and hide each other's
-    // projection / selection phases; one wave when there are too few tokens to fill the chip
-    const int nw = tokens >= 8192 ? 2 : 1;
+    // four waves (64 tokens) per workgroup: the waves share the work of bringing in the router
+    // matrix, which every workgroup reads in full
+    constexpr int nw = 4;
     const int tok = 16 * nw;
     const int blocks = (int)((tokens + tok - 1) / tok);
     const size_t smem = router_mfma_smem_bytes((int)E, (int)K, tok);
@@ -404,12 +443,9 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
         (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws);                   \
   }
-#define JT_ROUTER_CASE(NB)        \
-  case NB * 16:                   \
-    if (nw == 2)                  \
-      JT_ROUTER_LAUNCH(NB, 2)     \
-    else                          \
-      JT_ROUTER_LAUNCH(NB, 1)     \
+#define JT_ROUTER_CASE(NB)    \
+  case NB * 16:               \
+    JT_ROUTER_LAUNCH(NB, nw)  \
     break;
       switch ((int)E) {
         JT_ROUTER_CASE(1)

@@ -126,3 +126,30 @@ def test_bf16_layer_with_fp32_params_matches_oracle(gpu):
     assert same.mean() > 0.98
     err = np.max(np.abs(got.reshape(-1, 64)[same] - ref.y.reshape(-1, 64)[same])) / np.max(np.abs(ref.y))
     assert err <= 2e-2
+
+
+def test_graph_replay_matches_eager_on_every_replay(gpu):
+    """The captured layer gives the eager result on each of several replays with fresh inputs, with
+    eager work and synchronisations between the replays."""
+    from oracle import moe_oracle as O
+    from research_amd import ops
+    from research_amd.graph import GraphedLayer
+
+    inp = O.make_inputs("C5", seed=0)
+    cfg = inp["cfg"]
+    bf = lambda a: torch.from_numpy(a).to(gpu).to(torch.bfloat16).contiguous()
+    params = (bf(inp["w_router"]), torch.from_numpy(inp["expert_bias"]).to(gpu), bf(inp["gate"]), bf(inp["up"]),
+              bf(inp["down"]))
+    x0 = bf(inp["x"].reshape(-1, cfg["H"]))
+    layer = GraphedLayer(x0, *params, cfg["K"], 1.0)
+    gen = torch.Generator(device=gpu).manual_seed(5)
+    for i in range(4):
+        x = torch.randn(x0.shape, device=gpu, generator=gen).to(torch.bfloat16) if i else x0
+        eager = ops.moe_forward(x, *params, cfg["K"], 1.0)
+        torch.cuda.synchronize()
+        got = layer.replay(x)
+        torch.cuda.synchronize()
+        assert torch.equal(got.y, eager.y), f"replay {i}"
+        assert torch.equal(got.expert_ids, eager.expert_ids) and torch.equal(got.weights, eager.weights)
+        assert torch.equal(got.expert_counts, eager.expert_counts) and torch.equal(got.inverse, eager.inverse)
+        (eager.y.float() * 2).sum().item()  # unrelated eager work between the replays
