@@ -339,8 +339,9 @@ using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16>;
 using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64>;
 // Few rows per group (decode-sized batches): the layer streams every expert matrix once and
 // is bound by HBM, so the tiles are only 64 rows tall to keep the padded-row MFMA work below
-// the time the weights take to arrive.  Two workgroups fit the LDS of one CU.
+// the time the weights take to arrive.  Several workgroups share a CU, so that one computes
+// while another waits for its tiles.
 using GateUpSmallCfg = DmaGemmCfg<64, 128, 64, 2, 4, true, 2, 16>;
-using DownSmallCfg = DmaGemmCfg<64, 256, 64, 2, 4, false, 2, 16>;
+using DownSmallCfg = DmaGemmCfg<64, 256, 32, 1, 4, false, 2, 16>;  // four workgroups of four waves per CU
 
 }  // namespace jtmoe

@@ -398,6 +398,18 @@ static void time_backward() {
   }
 }
 
+// decode-sized batch: 8 rows per group, bound by streaming the expert matrices
+static void time_decode() {
+  Problem g = make(64, 512, 2048, 1408, 8, false, 0, 1.0f);
+  timeit<GateUpCfg>("gate/up 64 groups, 256-row tiles", g, 20);
+  timeit<GateUpSmallCfg>("gate/up 64 groups, 64-row tiles", g, 20);
+  release(g);
+  Problem d = make(64, 512, 1408, 2048, 9, false, 0, 1.0f);
+  timeit<DownCfg>("down 64 groups, 256-row tiles", d, 20);
+  timeit<DownSmallCfg>("down 64 groups, 64-row tiles", d, 20);
+  release(d);
+}
+
 int main(int argc, char** argv) {
   bool ok = true;
   {
@@ -451,6 +463,7 @@ int main(int argc, char** argv) {
     release(p);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_backward")) time_backward();
+  if (ok && argc > 1 && !strcmp(argv[1], "time_decode")) time_decode();
   if (ok && argc > 1 && !strcmp(argv[1], "time")) {
     for (float scale : {1.0f, 0.0f}) {
       printf("-- operand data: %s\n", scale > 0 ? "N(0,1) activations, N(0,0.05) weights" : "all zeros");
@@ -462,15 +475,7 @@ int main(int argc, char** argv) {
       release(d);
     }
     time_backward();
-    // decode-sized batch: 8 rows per group, bound by streaming the expert matrices
-    Problem g = make(64, 512, 2048, 1408, 8, false, 0, 1.0f);
-    timeit<GateUpCfg>("gate/up 64 groups, 256-row tiles", g, 20);
-    timeit<GateUpSmallCfg>("gate/up 64 groups, 64-row tiles", g, 20);
-    release(g);
-    Problem d = make(64, 512, 1408, 2048, 9, false, 0, 1.0f);
-    timeit<DownCfg>("down 64 groups, 256-row tiles", d, 20);
-    timeit<DownSmallCfg>("down 64 groups, 64-row tiles", d, 20);
-    release(d);
+    time_decode();
   }
   printf(ok ? "PASS\n" : "FAIL\n");
   return ok ? 0 : 1;
