@@ -200,6 +200,7 @@ def main() -> int:
     parser.add_argument("--cpu-sample-tokens", type=int, default=2048)
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-train", action="store_true", help="skip the forward+backward timing")
+    parser.add_argument("--no-block", action="store_true", help="skip the decoder-block and graph-replay timings")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: the layer runs with every expert local and no collective; "
@@ -385,9 +386,10 @@ def main() -> int:
         "roofline": roofline,
         "stages": stages,
     }
-    if T <= 2048:
-        line["graph_replay"] = graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, max(args.steps, 50))
-    line["block"] = block_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, ms_per_step)
+    if not args.no_block:
+        if T <= 2048:
+            line["graph_replay"] = graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, max(args.steps, 50))
+        line["block"] = block_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, ms_per_step)
     if not args.no_train:
         line["train"] = train_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, work)
     if not args.no_cpu_baseline:

@@ -315,7 +315,7 @@ int jtmoe_experts_backward(const void* x, const void* dy,
                            void* workspace, size_t workspace_bytes, void* stream);
 
 /* VJP of SharedSwiGLU.__call__ (moe.py:361-364): dx [T, H], d_gate, d_up [H, Is], d_down [Is, H]. */
-size_t jtmoe_shared_backward_workspace_bytes(int64_t T, int64_t Is, int dtype);
+size_t jtmoe_shared_backward_workspace_bytes(int64_t T, int64_t H, int64_t Is, int dtype);
 int jtmoe_shared_backward(const void* x, const void* dy,
                           const void* gate, const void* up, const void* down,
                           const void* gate_pre, const void* up_pre,
@@ -330,7 +330,7 @@ int jtmoe_shared_backward(const void* x, const void* dy,
  * selection itself and the expert bias carry no gradient (moe.py:139-140).
  *   dx [T, H], d_w_router [H, E].
  */
-size_t jtmoe_router_backward_workspace_bytes(int64_t T, int64_t E, int dtype);
+size_t jtmoe_router_backward_workspace_bytes(int64_t T, int64_t H, int64_t E, int dtype);
 int jtmoe_router_backward(const void* x, const void* w_router,
                           const float* scores, const int32_t* expert_ids,
                           const void* d_weights, const float* d_scores, double route_scale,

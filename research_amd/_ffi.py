@@ -79,9 +79,9 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_ptr] * 12 + [c_i64] * 5 + [c_int] + [c_ptr] * 6 + [c_ptr, c_size, c_ptr],
     ),
-    "jtmoe_shared_backward_workspace_bytes": (c_size, [c_i64, c_i64, c_int]),
+    "jtmoe_shared_backward_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_int]),
     "jtmoe_shared_backward": (c_int, [c_ptr] * 7 + [c_i64] * 3 + [c_int] + [c_ptr] * 4 + [c_ptr, c_size, c_ptr]),
-    "jtmoe_router_backward_workspace_bytes": (c_size, [c_i64, c_i64, c_int]),
+    "jtmoe_router_backward_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_int]),
     "jtmoe_router_backward": (
         c_int,
         [c_ptr] * 6 + [c_dbl] + [c_i64] * 4 + [c_int] + [c_ptr] * 2 + [c_ptr, c_size, c_ptr],

@@ -211,16 +211,35 @@ ExpertsBwdWs carve_experts(void* base, int64_t A, int64_t H, int64_t I, int dtyp
 }
 
 struct SharedBwdWs {
-  void *dg, *du, *hw;
+  void *dg, *du, *hw, *split;
   size_t total;
 };
-SharedBwdWs carve_shared(void* base, int64_t T, int64_t Is, int dtype) {
+SharedBwdWs carve_shared(void* base, int64_t T, int64_t H, int64_t Is, int dtype) {
   Carver c{static_cast<unsigned char*>(base)};
   const size_t b = dtype_bytes(dtype);
   SharedBwdWs w;
   w.dg = c.take((size_t)T * Is * b);
   w.du = c.take((size_t)T * Is * b);
   w.hw = c.take((size_t)T * Is * b);
+  // partial sums of the two weight-gradient reductions (used one after the other)
+  const size_t down_split = gemm_tn_split_bytes(dtype, T, Is, H, false);
+  const size_t gate_up_split = gemm_tn_split_bytes(dtype, T, H, Is, true);
+  const size_t split = down_split > gate_up_split ? down_split : gate_up_split;
+  w.split = split ? c.take(split) : nullptr;
+  w.total = c.used;
+  return w;
+}
+
+struct RouterBwdWs {
+  void *d_logits, *split;
+  size_t total;
+};
+RouterBwdWs carve_router(void* base, int64_t T, int64_t H, int64_t E, int dtype) {
+  Carver c{static_cast<unsigned char*>(base)};
+  RouterBwdWs w;
+  w.d_logits = c.take((size_t)T * E * dtype_bytes(dtype));
+  const size_t split = gemm_tn_split_bytes(dtype, T, H, E, false);
+  w.split = split ? c.take(split) : nullptr;
   w.total = c.used;
   return w;
 }
@@ -272,10 +291,10 @@ int shared_backward_impl(const void* x, const void* dy, const void* gate, const 
            : run_swiglu_backward<float>(ws.dg, gate_pre, up_pre, nullptr, nullptr, T, Is, ws.du, ws.hw, nullptr, s);
   if (rc) return rc;
   rc = launch_gemm_tn(dtype, ws.hw, dy, nullptr, d_down, nullptr, nullptr, nullptr, T, Is, H, 1, nullptr, 1, false,
-                      false, 0, s);
+                      false, 0, s, ws.split);
   if (rc) return rc;
   rc = launch_gemm_tn(dtype, x, ws.dg, ws.du, d_gate, d_up, nullptr, nullptr, T, H, Is, 1, nullptr, 1, false, false, 0,
-                      s);
+                      s, ws.split);
   if (rc) return rc;
   rc = launch_gemm_nt(dtype, ws.dg, ws.du, gate, up, dx, nullptr, nullptr, T, Is, H, 1, nullptr, 1, 0, 2, s);
   if (rc) return rc;
@@ -284,8 +303,9 @@ int shared_backward_impl(const void* x, const void* dy, const void* gate, const 
 
 int router_backward_impl(const void* x, const void* router_weight, const float* scores, const int32_t* ids,
                          const void* d_weights, const float* d_scores, double route_scale, int64_t T, int64_t H,
-                         int64_t E, int64_t K, int dtype, void* dx, void* d_router_weight, void* d_logits,
+                         int64_t E, int64_t K, int dtype, void* dx, void* d_router_weight, const RouterBwdWs& ws,
                          hipStream_t s) {
+  void* const d_logits = ws.d_logits;
   const unsigned grid = (unsigned)((T + 3) / 4);
   if (T == 0) {
     // no tokens: the weight gradient is all zeros, which the empty reduction below writes
@@ -301,7 +321,7 @@ int router_backward_impl(const void* x, const void* router_weight, const float* 
   if (rc) return rc;
   // dW_r [H, E] = x^T @ dlogits;  dx [T, H] = dlogits @ W_r^T  (W_r is [H, E]: N = H rows of length K = E)
   rc = launch_gemm_tn(dtype, x, d_logits, nullptr, d_router_weight, nullptr, nullptr, nullptr, T, H, E, 1, nullptr, 1,
-                      false, false, 0, s);
+                      false, false, 0, s, ws.split);
   if (rc) return rc;
   return launch_gemm_nt(dtype, d_logits, nullptr, router_weight, nullptr, dx, nullptr, nullptr, T, E, H, 1, nullptr, 1,
                         0, 1, s);
@@ -362,9 +382,9 @@ extern "C" int jtmoe_experts_backward(const void* x, const void* dy, const int32
   return jtmoe_combine(ws.dxp, inverse, ws.ones, dx_extra, T, H, K, dtype, dx, stream);
 }
 
-extern "C" size_t jtmoe_shared_backward_workspace_bytes(int64_t T, int64_t Is, int dtype) {
-  if (T < 0 || Is <= 0 || !dtype_ok(dtype)) return 0;
-  return carve_shared(nullptr, T, Is, dtype).total;
+extern "C" size_t jtmoe_shared_backward_workspace_bytes(int64_t T, int64_t H, int64_t Is, int dtype) {
+  if (T < 0 || H <= 0 || Is <= 0 || !dtype_ok(dtype)) return 0;
+  return carve_shared(nullptr, T, H, Is, dtype).total;
 }
 
 extern "C" int jtmoe_shared_backward(const void* x, const void* dy, const void* gate, const void* up, const void* down,
@@ -376,7 +396,7 @@ extern "C" int jtmoe_shared_backward(const void* x, const void* dy, const void* 
   if (rc) return rc;
   JT_REQUIRE(gate && up && down && d_gate && d_up && d_down, "shared_backward: null weight pointer");
   if (T > 0) JT_REQUIRE(x && dy && gate_pre && up_pre && dx, "shared_backward: null pointer argument");
-  const SharedBwdWs ws = carve_shared(workspace, T, Is, dtype);
+  const SharedBwdWs ws = carve_shared(workspace, T, H, Is, dtype);
   if (T > 0 && (workspace == nullptr || workspace_bytes < ws.total))
     return fail(JTMOE_EWORKSPACE, "shared_backward: workspace of %zu bytes given, %zu needed", workspace_bytes,
                 ws.total);
@@ -384,9 +404,9 @@ extern "C" int jtmoe_shared_backward(const void* x, const void* dy, const void* 
                               as_stream(stream));
 }
 
-extern "C" size_t jtmoe_router_backward_workspace_bytes(int64_t T, int64_t E, int dtype) {
-  if (T < 0 || E <= 0 || !dtype_ok(dtype)) return 0;
-  return align_up((size_t)T * E * dtype_bytes(dtype), 256);
+extern "C" size_t jtmoe_router_backward_workspace_bytes(int64_t T, int64_t H, int64_t E, int dtype) {
+  if (T < 0 || H <= 0 || E <= 0 || !dtype_ok(dtype)) return 0;
+  return carve_router(nullptr, T, H, E, dtype).total;
 }
 
 extern "C" int jtmoe_router_backward(const void* x, const void* router_weight, const float* scores,
@@ -399,19 +419,20 @@ extern "C" int jtmoe_router_backward(const void* x, const void* router_weight, c
   if (rc) return rc;
   JT_REQUIRE(router_weight && d_router_weight, "router_backward: null weight pointer");
   if (T > 0) JT_REQUIRE(x && scores && expert_ids && d_weights && dx, "router_backward: null pointer argument");
-  const size_t need = jtmoe_router_backward_workspace_bytes(T, E, dtype);
-  if (T > 0 && (workspace == nullptr || workspace_bytes < need))
-    return fail(JTMOE_EWORKSPACE, "router_backward: workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+  const RouterBwdWs ws = carve_router(workspace, T, H, E, dtype);
+  if (T > 0 && (workspace == nullptr || workspace_bytes < ws.total))
+    return fail(JTMOE_EWORKSPACE, "router_backward: workspace of %zu bytes given, %zu needed", workspace_bytes,
+                ws.total);
   return router_backward_impl(x, router_weight, scores, expert_ids, d_weights, d_scores, route_scale, T, H, E, K,
-                              dtype, dx, d_router_weight, workspace, as_stream(stream));
+                              dtype, dx, d_router_weight, ws, as_stream(stream));
 }
 
 extern "C" size_t jtmoe_moe_backward_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
                                                      int dtype) {
   if (T < 0 || K <= 0 || H <= 0 || I <= 0 || E <= 0 || Is < 0 || !dtype_ok(dtype)) return 0;
   size_t total = carve_experts(nullptr, T * K, H, I, dtype).total;
-  if (Is > 0) total += carve_shared(nullptr, T, Is, dtype).total;
-  total += jtmoe_router_backward_workspace_bytes(T, E, dtype);
+  if (Is > 0) total += carve_shared(nullptr, T, H, Is, dtype).total;
+  total += carve_router(nullptr, T, H, E, dtype).total;
   total += 3 * align_up((size_t)T * H * dtype_bytes(dtype), 256);  // dx of the shared experts, of the router, their sum
   total += align_up((size_t)T * K * dtype_bytes(dtype), 256);      // gradient of the route weights
   return total;
@@ -449,8 +470,8 @@ extern "C" int jtmoe_moe_backward(const void* x, const void* dy, const float* d_
   Carver c{static_cast<unsigned char*>(workspace)};
   const ExpertsBwdWs ews = carve_experts(c.take(carve_experts(nullptr, T * K, H, I, dtype).total), T * K, H, I, dtype);
   SharedBwdWs sws{};
-  if (Is > 0) sws = carve_shared(c.take(carve_shared(nullptr, T, Is, dtype).total), T, Is, dtype);
-  void* d_logits = c.take(jtmoe_router_backward_workspace_bytes(T, E, dtype));
+  if (Is > 0) sws = carve_shared(c.take(carve_shared(nullptr, T, H, Is, dtype).total), T, H, Is, dtype);
+  const RouterBwdWs rws = carve_router(c.take(carve_router(nullptr, T, H, E, dtype).total), T, H, E, dtype);
   const size_t th = (size_t)T * H * dtype_bytes(dtype);
   void* dx_shared = c.take(th);
   void* dx_router = c.take(th);
@@ -466,7 +487,7 @@ extern "C" int jtmoe_moe_backward(const void* x, const void* dy, const float* d_
     if (rc) return rc;
   }
   rc = router_backward_impl(x, router_weight, scores, expert_ids, d_weights, d_scores, route_scale, T, H, E, K, dtype,
-                            dx_router, d_router_weight, d_logits, s);
+                            dx_router, d_router_weight, rws, s);
   if (rc) return rc;
   if (T == 0) return JTMOE_OK;
   const void* extra = dx_router;

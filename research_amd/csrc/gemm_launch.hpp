@@ -17,9 +17,13 @@ int launch_gemm_nt(int dtype, const void* a0, const void* a1, const void* b0, co
 // C_i[e] = P[rows of group e, :]^T @ D_i[rows of group e, :]     (i = 0, and 1 if d1 is given)
 //   P: [rows, KA], D_i: [rows, N]; either may instead be [gathered_rows, .] read through row_map
 //   C_i: [E, KA, N]; an empty group yields zeros
+//   split_ws: scratch of gemm_tn_split_bytes(...) bytes, or nullptr.  With it, a one-group call whose
+//   output has too few tiles to fill the chip is run as partial sums over runs of rows (float32, in
+//   split_ws) that a second kernel adds up in a fixed order.
 int launch_gemm_tn(int dtype, const void* p, const void* d0, const void* d1, void* c0, void* c1,
                    const int32_t* group_sizes, const int32_t* offsets, int64_t rows, int64_t KA, int64_t N, int64_t E,
                    const int32_t* row_map, int row_div, bool p_gather, bool d_gather, int64_t gathered_rows,
-                   hipStream_t stream);
+                   hipStream_t stream, void* split_ws = nullptr);
+size_t gemm_tn_split_bytes(int dtype, int64_t rows, int64_t KA, int64_t N, bool dual);
 
 }  // namespace jtmoe

@@ -188,10 +188,43 @@ int launch_gemm_nt(int dtype, const void* a0, const void* a1, const void* b0, co
 }
 
 namespace {
+
+// out[i] = round(sum over s of partial[s][i]), s ascending
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ partial, int splits,
+                                                              size_t n, uint16_t* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float acc = 0.0f;
+  for (int s = 0; s < splits; ++s) acc += partial[(size_t)s * n + i];
+  out[i] = (uint16_t)f32_to_bf16_bits(acc);
+}
+
+struct SplitPlan {
+  int splits;  // 0: do not split
+  int chunk;   // rows per run, a multiple of the k step
+};
+
+// A one-group reduction is split when its output tiles cannot occupy the chip and there are
+// enough rows to share out.
+template <typename Cfg>
+SplitPlan split_plan(int64_t rows, int64_t KA, int64_t N) {
+  const int64_t tiles = ((KA + Cfg::BMO - 1) / Cfg::BMO) * ((N + Cfg::BNO - 1) / Cfg::BNO);
+  SplitPlan p{0, 0};
+  if (tiles >= 200 || rows < 2048) return p;
+  int64_t splits = (512 + tiles - 1) / tiles;
+  if (splits > rows / 256) splits = rows / 256;
+  if (splits < 2) return p;
+  const int64_t chunk = ((rows + splits - 1) / splits + 63) / 64 * 64;
+  p.splits = (int)((rows + chunk - 1) / chunk);
+  p.chunk = (int)chunk;
+  return p;
+}
+
 template <typename Cfg>
 int launch_tn_fast(const void* p, const void* d0, const void* d1, void* c0, void* c1, const int32_t* group_sizes,
                    const int32_t* offsets, int64_t rows, int64_t KA, int64_t N, int64_t E, const int32_t* row_map,
-                   int row_div, bool p_gather, bool d_gather, int64_t gathered_rows, hipStream_t stream) {
+                   int row_div, bool p_gather, bool d_gather, int64_t gathered_rows, hipStream_t stream,
+                   void* split_ws) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   auto kernel = grouped_gemm_tn_kernel<Cfg>;
@@ -199,12 +232,28 @@ int launch_tn_fast(const void* p, const void* d0, const void* d1, void* c0, void
   if (attr_err != hipSuccess)
     return fail(JTMOE_ELAUNCH, "grouped gemm (tn): hipFuncSetAttribute: %s", hipGetErrorString(attr_err));
   const int64_t mt = (KA + Cfg::BMO - 1) / Cfg::BMO, nt = (N + Cfg::BNO - 1) / Cfg::BNO;
+  SplitPlan plan{0, 0};
+  if (split_ws != nullptr && group_sizes == nullptr && !p_gather && !d_gather) plan = split_plan<Cfg>(rows, KA, N);
+  if (plan.splits > 0) {
+    const size_t n = (size_t)KA * N;
+    float* part0 = static_cast<float*>(split_ws);
+    float* part1 = part0 + (size_t)plan.splits * n;
+    const int64_t grid = gemm_grid(plan.splits * mt, nt);
+    kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
+        static_cast<const uint16_t*>(p), static_cast<const uint16_t*>(d0), static_cast<const uint16_t*>(d1),
+        reinterpret_cast<uint16_t*>(part0), reinterpret_cast<uint16_t*>(part1), nullptr, nullptr, plan.splits,
+        (int)rows, (int)KA, (int)N, (int)mt, (int)nt, nullptr, 1, 0, 0, 0, plan.chunk);
+    const unsigned rgrid = (unsigned)((n + 255) / 256);
+    reduce_partials_kernel<<<rgrid, 256, 0, stream>>>(part0, plan.splits, n, static_cast<uint16_t*>(c0));
+    if (Cfg::kDual) reduce_partials_kernel<<<rgrid, 256, 0, stream>>>(part1, plan.splits, n, static_cast<uint16_t*>(c1));
+    return JTMOE_OK;
+  }
   const int64_t grid = gemm_grid(E * mt, nt);
   if (grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm (tn): grid too large");
   kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
       static_cast<const uint16_t*>(p), static_cast<const uint16_t*>(d0), static_cast<const uint16_t*>(d1),
       static_cast<uint16_t*>(c0), static_cast<uint16_t*>(c1), group_sizes, offsets, (int)E, (int)rows, (int)KA,
-      (int)N, (int)mt, (int)nt, row_map, row_div, p_gather ? 1 : 0, d_gather ? 1 : 0, (int)gathered_rows);
+      (int)N, (int)mt, (int)nt, row_map, row_div, p_gather ? 1 : 0, d_gather ? 1 : 0, (int)gathered_rows, 0);
   return JTMOE_OK;
 }
 }  // namespace
@@ -212,7 +261,7 @@ int launch_tn_fast(const void* p, const void* d0, const void* d1, void* c0, void
 int launch_gemm_tn(int dtype, const void* p, const void* d0, const void* d1, void* c0, void* c1,
                    const int32_t* group_sizes, const int32_t* offsets, int64_t rows, int64_t KA, int64_t N, int64_t E,
                    const int32_t* row_map, int row_div, bool p_gather, bool d_gather, int64_t gathered_rows,
-                   hipStream_t stream) {
+                   hipStream_t stream, void* split_ws) {
   const bool dual = d1 != nullptr;
   const int64_t p_rows = p_gather ? gathered_rows : rows, d_rows = d_gather ? gathered_rows : rows;
   const bool fast = dtype == JTMOE_BF16 && KA % 8 == 0 && N % 8 == 0 && p_rows * KA < kOperandLimit &&
@@ -221,9 +270,9 @@ int launch_gemm_tn(int dtype, const void* p, const void* d0, const void* d1, voi
   if (fast) {
     if (dual)
       return launch_tn_fast<WgradDualCfg>(p, d0, d1, c0, c1, group_sizes, offsets, rows, KA, N, E, row_map, row_div,
-                                          p_gather, d_gather, gathered_rows, stream);
+                                          p_gather, d_gather, gathered_rows, stream, split_ws);
     return launch_tn_fast<WgradCfg>(p, d0, nullptr, c0, nullptr, group_sizes, offsets, rows, KA, N, E, row_map,
-                                    row_div, p_gather, d_gather, gathered_rows, stream);
+                                    row_div, p_gather, d_gather, gathered_rows, stream, split_ws);
   }
   const int64_t mt = (KA + QB - 1) / QB, nt = (N + QB - 1) / QB;
   if (E * mt * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm (tn): grid too large");
@@ -240,6 +289,13 @@ int launch_gemm_tn(int dtype, const void* p, const void* d0, const void* d1, voi
           (int)rows, (int)KA, (int)N, (int)mt, (int)nt, row_map, row_div, p_gather ? 1 : 0, d_gather ? 1 : 0);
   }
   return JTMOE_OK;
+}
+
+size_t gemm_tn_split_bytes(int dtype, int64_t rows, int64_t KA, int64_t N, bool dual) {
+  if (dtype != JTMOE_BF16 || KA % 8 != 0 || N % 8 != 0) return 0;
+  const SplitPlan plan = dual ? split_plan<WgradDualCfg>(rows, KA, N) : split_plan<WgradCfg>(rows, KA, N);
+  if (plan.splits == 0) return 0;
+  return align_up((size_t)plan.splits * KA * N * sizeof(float) * (dual ? 2 : 1), 256);
 }
 
 }  // namespace jtmoe

@@ -239,7 +239,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
     const uint16_t* __restrict__ P, const uint16_t* __restrict__ D0, const uint16_t* __restrict__ D1,
     uint16_t* __restrict__ C0, uint16_t* __restrict__ C1, const int32_t* __restrict__ group_sizes,
     const int32_t* __restrict__ offsets, int E, int dense_rows, int KA, int N, int mtiles_o, int ntiles_o,
-    const int32_t* __restrict__ row_map, int row_div, int p_gather, int d_gather, int gathered_rows) {
+    const int32_t* __restrict__ row_map, int row_div, int p_gather, int d_gather, int gathered_rows,
+    int split_chunk) {
   constexpr int BMO = Cfg::BMO, BNO = Cfg::BNO, BK = Cfg::BK, NT = Cfg::NT;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   constexpr bool kDual = Cfg::kDual;
@@ -258,10 +259,16 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   const int mt = in_e - nt * mtiles_o;
   const int m0 = mt * BMO, n0 = nt * BNO;
 
+  // split_chunk > 0 (one dense group only): "group" e is the e-th run of split_chunk rows, and the
+  // outputs are float32 partial sums [E, KA, N] that the caller adds up in a fixed order.  This
+  // gives a reduction over many rows into a small matrix enough workgroups to fill the chip.
   int row0, rows;
   if (group_sizes) {
     row0 = __builtin_amdgcn_readfirstlane(offsets[e]);
     rows = __builtin_amdgcn_readfirstlane(group_sizes[e]);
+  } else if (split_chunk > 0) {
+    row0 = e * split_chunk;
+    rows = max(0, min(split_chunk, dense_rows - row0));
   } else {
     row0 = 0;
     rows = dense_rows;
@@ -399,8 +406,28 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   wait_vmcnt<0>();
   __syncthreads();
 
-  // epilogue: per matrix, each wave parks its WM x WNO block in LDS and streams it out in rows
   constexpr int TNO = Cfg::TNO, WNO = Cfg::WNO, CS = Cfg::CS;
+  if (split_chunk > 0) {
+    // float32 partial sums straight from the accumulators: for a fixed i the 32 lanes of a half
+    // wave write 128 contiguous bytes of one row
+#pragma unroll
+    for (int which = 0; which < (kDual ? 2 : 1); ++which) {
+      float* const Cm = reinterpret_cast<float*>(which ? C1 : C0) + (size_t)e * KA * N;
+#pragma unroll
+      for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int jj = 0; jj < TNO; ++jj) {
+          const int col = n0 + wn * WNO + jj * 32 + (lane & 31);
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int r = m0 + wm * WM + mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+            if (r < KA && col < N) Cm[(size_t)r * N + col] = acc[mi][jj + which * (TN / 2)][i];
+          }
+        }
+    }
+    return;
+  }
+  // epilogue: per matrix, each wave parks its WM x WNO block in LDS and streams it out in rows
   uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
   constexpr int CPR_OUT = WNO / 8;
   constexpr int OUT_CHUNKS = WM * CPR_OUT;

@@ -278,7 +278,7 @@ static void launch_tn(Problem& p, const uint16_t* D0, const uint16_t* D1, uint16
   const int groups = dense ? 1 : p.E;
   kernel<<<(unsigned)gemm_grid(groups * mt, nt), Cfg::NT, Cfg::SMEM_BYTES>>>(
       p.A, D0, D1, C0, C1, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, groups, p.rows, p.K, p.N, (int)mt,
-      (int)nt, p.dmap, p.top_k > 0 ? p.top_k : 1, p_gather, d_gather, p.a_rows);
+      (int)nt, p.dmap, p.top_k > 0 ? p.top_k : 1, p_gather, d_gather, p.a_rows, 0);
 }
 
 // which operand goes through the row map: 0 none, 1 the transposed one (P), 2 the other (D)

@@ -144,7 +144,7 @@ def shared_backward(x, dy, gate, up, down, residuals: ExpertResiduals):
     dx = torch.empty_like(x)
     d_gate, d_up, d_down = torch.empty_like(gate), torch.empty_like(up), torch.empty_like(down)
     lib = _lib()
-    ws = _workspace(lib.jtmoe_shared_backward_workspace_bytes(tokens, inter, _code(x.dtype)), dev)
+    ws = _workspace(lib.jtmoe_shared_backward_workspace_bytes(tokens, hidden, inter, _code(x.dtype)), dev)
     status = lib.jtmoe_shared_backward(
         _ptr(x), _ptr(dy), _ptr(gate), _ptr(up), _ptr(down), _ptr(residuals.gate_pre), _ptr(residuals.up_pre),
         tokens, hidden, inter, _code(x.dtype), _ptr(dx), _ptr(d_gate), _ptr(d_up), _ptr(d_down),
@@ -176,7 +176,7 @@ def router_backward(x, w_router, scores, expert_ids, d_weights, d_scores=None, r
     dx = torch.empty_like(x)
     d_w = torch.empty_like(w_router)
     lib = _lib()
-    ws = _workspace(lib.jtmoe_router_backward_workspace_bytes(tokens, experts, _code(x.dtype)), dev)
+    ws = _workspace(lib.jtmoe_router_backward_workspace_bytes(tokens, hidden, experts, _code(x.dtype)), dev)
     status = lib.jtmoe_router_backward(
         _ptr(x), _ptr(w_router), _ptr(scores), _ptr(expert_ids), _ptr(d_weights), _ptr(d_scores), float(route_scale),
         tokens, hidden, experts, top_k, _code(x.dtype), _ptr(dx), _ptr(d_w), ws.data_ptr(), ws.numel(), _stream(dev),

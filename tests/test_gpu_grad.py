@@ -92,7 +92,9 @@ def test_expert_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, inte
         assert not got.d_gate[e].any() and not got.d_up[e].any() and not got.d_down[e].any()
 
 
-@pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16")])
+# the 4096-token cases take the path that splits a long one-group reduction into partial sums
+@pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16"),
+                                                       (4096, 512, 704, "bf16")])
 def test_shared_gradients_match_oracle(gpu, tokens, hidden, inter, dtype):
     rng = np.random.default_rng(7)
     std = 0.02 if hidden >= 512 else 0.2
@@ -115,7 +117,7 @@ def test_shared_gradients_match_oracle(gpu, tokens, hidden, inter, dtype):
 
 @pytest.mark.parametrize("tokens,hidden,experts,top_k,dtype,with_scores",
                          [(6, 5, 7, 3, "f32", True), (300, 256, 64, 8, "bf16", True), (129, 72, 10, 2, "bf16", False),
-                          (512, 2048, 128, 8, "bf16", True)])
+                          (512, 2048, 128, 8, "bf16", True), (4100, 256, 64, 8, "bf16", True)])
 def test_router_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, dtype, with_scores):
     rng = np.random.default_rng(11)
     x = rng.standard_normal((tokens, hidden)).astype(np.float32)
