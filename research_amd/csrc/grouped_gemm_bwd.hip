@@ -210,7 +210,7 @@ template <typename Cfg>
 SplitPlan split_plan(int64_t rows, int64_t KA, int64_t N) {
   const int64_t tiles = ((KA + Cfg::BMO - 1) / Cfg::BMO) * ((N + Cfg::BNO - 1) / Cfg::BNO);
   SplitPlan p{0, 0};
-  if (tiles >= 200 || rows < 2048) return p;
+  if (tiles > 128 || rows < 2048) return p;
   int64_t splits = (512 + tiles - 1) / tiles;
   if (splits > rows / 256) splits = rows / 256;
   if (splits < 2) return p;
