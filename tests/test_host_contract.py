@@ -74,3 +74,22 @@ def test_jax_ffi_stub_fails_loudly_without_jax():
     assert set(jax_ffi.TARGETS.values()) == {
         "JaxtitanMoeForward", "JaxtitanMoeRouter", "JaxtitanMoeDispatch", "JaxtitanMoeGroupedSwiglu",
         "JaxtitanMoeCombine"}
+
+
+def test_training_and_block_operators_refuse_cpu_tensors_and_bad_shapes():
+    from research_amd import grad
+
+    x, dy = torch.zeros((4, 8)), torch.zeros((4, 8))
+    gate = up = torch.zeros((2, 8, 16))
+    down = torch.zeros((2, 16, 8))
+    with pytest.raises(ContractError, match="GPU"):
+        grad.shared_swiglu_train(x, gate[0], up[0], down[0])
+    with pytest.raises(ContractError, match="GPU"):
+        grad.router_backward(x, torch.zeros((8, 2)), torch.zeros((4, 2)), torch.zeros((4, 1), dtype=torch.int32),
+                             torch.zeros((4, 1)))
+    with pytest.raises(ContractError, match="GPU"):
+        ops.rmsnorm(x, torch.ones(8))
+    with pytest.raises(ContractError, match="GPU"):
+        ops.ffn_block_forward(x, torch.ones(8), torch.ones(8), 1e-6, torch.zeros((8, 2)), None, gate, up, down, 1)
+    with pytest.raises(ContractError, match="GPU"):
+        grad.moe_forward_train(x, torch.zeros((8, 2)), None, gate, up, down, 1)
