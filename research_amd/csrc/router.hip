@@ -114,13 +114,12 @@ __device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, in
 
 // Everything after the logits tile is in LDS.  `T` is the output element type of
 // the weights.
-template <typename T, int NW>
+template <typename T, int kRouterTokens, int kRouterThreads>
 __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ bias_g, int t0, int tokens,
                                 int E, int K, float route_scale, int32_t* __restrict__ ids_out,
                                 T* __restrict__ weights_out, float* __restrict__ scores_out,
                                 float* __restrict__ logits_out, RouterScratch g) {
 #pragma clang fp contract(off)
-  constexpr int kRouterTokens = 16 * NW, kRouterThreads = 64 * NW;
   const int tid = threadIdx.x;
   const int stride = E + 1;
   const int nrows = min(kRouterTokens, tokens - t0);
@@ -236,8 +235,8 @@ __global__ __launch_bounds__(256) void router_kernel(
     sm.tile[t * stride + e] = z;
   }
   __syncthreads();
-  router_epilogue<T, 4>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
-                        router_scratch(ws, E));
+  router_epilogue<T, 64, 256>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
+                              router_scratch(ws, E));
 }
 
 // ---------------------------------------------------------------------------
@@ -404,8 +403,135 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
     for (int i = 0; i < 4; ++i)
       sm.tile[(wave * 16 + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = round_to_bf16(acc[nb][i]);
   __syncthreads();
-  router_epilogue<bf16_raw, NW>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
-                                router_scratch(ws, E));
+  router_epilogue<bf16_raw, 16 * NW, 64 * NW>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores,
+                                              logits_out, router_scratch(ws, E));
+}
+
+// ---------------------------------------------------------------------------
+// The same projection with the k range of every staged chunk shared out over the four waves
+// of a workgroup: 16 tokens per workgroup, 128 k rows per LDS stage, wave w multiplying rows
+// [32 w, 32 w + 32) of each stage.  The four partial sums are added in wave order.  A workgroup
+// then runs H/128 short iterations instead of H/64 longer ones, and 16 tokens already make a
+// workgroup, so small batches spread over more CUs.
+// ---------------------------------------------------------------------------
+constexpr int kSplitKC = 128;
+constexpr int kSplitMaxTokens = 256;
+
+__host__ __device__ inline size_t router_split_red_offset(int E, int K) {
+  return (router_smem_bytes(E, K, 16) + 15) / 16 * 16;
+}
+__host__ __device__ inline size_t router_split_smem_bytes(int E, int K) {
+  const size_t w = (size_t)2 * kSplitKC * router_w_stride(E) * 2;
+  const size_t ep = router_split_red_offset(E, K) + (size_t)4 * 16 * (E + 1) * 4;
+  return w > ep ? w : ep;
+}
+
+template <int NB>
+__global__ __launch_bounds__(256) void router_mfma_split_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
+    int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
+    float* __restrict__ scores, float* __restrict__ logits_out, void* ws) {
+  constexpr int kThreads = 256, kTokens = 16;
+  constexpr int E = NB * 16;
+  constexpr int WS = E + 32;
+  constexpr int W_CHUNKS = kSplitKC * E / 8;
+  constexpr int CW = (W_CHUNKS + kThreads - 1) / kThreads;
+  constexpr int CPR = E / 8;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  uint16_t* const Ws = reinterpret_cast<uint16_t*>(smem_raw);  // [2][kSplitKC][WS]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int t0 = blockIdx.x * kTokens;
+  const int nrows = min(kTokens, tokens - t0);
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(x + (size_t)t0 * H), 0, nrows * H * 2, kBufferFlags);
+  // lane (m = lane%16, kg = lane/16) holds k = chunk*128 + wave*32 + kg*8 + [0,8) of token t0 + m
+  const int x_voff = ((lane & 15) * H + wave * 32 + (lane >> 4) * 8) * 2;
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(w), 0, H * E * 2, kBufferFlags);
+
+  constexpr int D = CW <= 8 ? 3 : 2;   // chunks in flight (register ring, chunk c in slot c % D)
+  constexpr int UNROLL = D == 3 ? 6 : 2;
+  u32x4_t a_ring[D], w_ring[D][CW];
+  f32x4_t acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[nb][i] = 0.0f;
+
+#define JT_LOAD(slot, k0)                                                                     \
+  {                                                                                           \
+    _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                          \
+      const int c = tid + i * kThreads;                                                       \
+      if (W_CHUNKS % kThreads == 0 || c < W_CHUNKS)                                           \
+        w_ring[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c * 16, (k0)*E * 2, 0); \
+    }                                                                                         \
+    a_ring[slot] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff, (k0)*2, 0);          \
+  }
+#define JT_STORE_W(slot, stage)                                                               \
+  _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                            \
+    const int c = tid + i * kThreads;                                                         \
+    if (W_CHUNKS % kThreads == 0 || c < W_CHUNKS) {                                           \
+      const int kr = c / CPR, nc = c - kr * CPR;                                              \
+      *reinterpret_cast<u32x4_t*>(Ws + ((stage)*kSplitKC + kr) * WS + nc * 8) = w_ring[slot][i]; \
+    }                                                                                         \
+  }
+
+  // transposing read: the 16-lane group kg reads rows wave*32 + kg*8 + 4*h + i/4, columns 4*(i%4)..
+  const int w_lane = (wave * 32 + (lane >> 4) * 8 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
+  const int nchunks = H / kSplitKC;
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nchunks) JT_LOAD(d, d * kSplitKC);
+  JT_STORE_W(0, 0);
+  __syncthreads();
+  for (int kc0 = 0; kc0 < nchunks; kc0 += UNROLL) {
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+      const int kc = kc0 + j;
+      if (kc < nchunks) {  // uniform over the workgroup
+        const int stage = j % 2, slot = j % D, next_slot = (j + 1) % D;
+        const uint16_t* wbase = Ws + stage * kSplitKC * WS + w_lane;
+        const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_ring[slot]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const uint16_t* p = wbase + nb * 16;
+          const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+          const s16x4_t hi =
+              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
+          const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
+        }
+        if (kc + 1 < nchunks) JT_STORE_W(next_slot, stage ^ 1);
+        if (kc + D < nchunks) JT_LOAD(slot, (kc + D) * kSplitKC);
+        __syncthreads();
+      }
+    }
+  }
+#undef JT_LOAD
+#undef JT_STORE_W
+
+  // partial sums of the four waves -> LDS, added in wave order, rounded to bf16 (the projection's
+  // output dtype); value i of lane l is token row 4*(l/16) + i, expert nb*16 + l%16
+  RouterSmem sm = router_smem(smem_raw, E, K, kTokens);
+  const int stride = E + 1;
+  float* const red = reinterpret_cast<float*>(smem_raw + router_split_red_offset(E, K));
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      red[(wave * kTokens + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = acc[nb][i];
+  __syncthreads();
+  for (int idx = tid; idx < kTokens * E; idx += kThreads) {
+    const int t = idx / E, e = idx - t * E;
+    float v = red[t * stride + e];
+#pragma unroll
+    for (int wv = 1; wv < 4; ++wv) v += red[(wv * kTokens + t) * stride + e];
+    sm.tile[t * stride + e] = round_to_bf16(v);
+  }
+  __syncthreads();
+  router_epilogue<bf16_raw, kTokens, kThreads>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores,
+                                               logits_out, router_scratch(ws, E));
 }
 
 template <typename KernelT>
@@ -425,6 +551,38 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
   const bool mfma = Elem<T>::is_bf16 && !kFromLogits && H % kRouterKC == 0 && H * E < ((int64_t)1 << 30) &&
                     (E == 16 || E == 32 || E == 64 || E == 128 || E == 256) && aligned16(x) && aligned16(w);
   if (mfma) {
+    // Up to a few hundred tokens the whole call is a handful of workgroups, each waiting on its own
+    // chain of chunks: the k-split kernel (16 tokens per workgroup, half as many and shorter
+    // iterations) is used; beyond that the 64-token workgroups stage the router matrix four times
+    // less often per token and win.
+    if (H % kSplitKC == 0 && tokens <= kSplitMaxTokens) {
+      const int blocks = (int)((tokens + 15) / 16);
+      const size_t smem = router_split_smem_bytes((int)E, (int)K);
+      if (smem > 160 * 1024)
+        return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
+      router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
+      if (tokens > 0) {
+#define JT_SPLIT_CASE(NB)                                                                                     \
+  case NB * 16: {                                                                                            \
+    auto kernel = router_mfma_split_kernel<NB>;                                                              \
+    int rc = set_max_smem(kernel, smem);                                                                     \
+    if (rc) return rc;                                                                                       \
+    kernel<<<blocks, 256, smem, stream>>>(                                                                   \
+        static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws);                   \
+  } break;
+        switch ((int)E) {
+          JT_SPLIT_CASE(1)
+          JT_SPLIT_CASE(2)
+          JT_SPLIT_CASE(4)
+          JT_SPLIT_CASE(8)
+          JT_SPLIT_CASE(16)
+        }
+#undef JT_SPLIT_CASE
+      }
+      router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
+      return check_launch("router");
+    }
     // four waves (64 tokens) per workgroup: the waves share the work of bringing in the router
     // matrix, which every workgroup reads in full
     constexpr int nw = 4;

