@@ -80,6 +80,51 @@ __device__ __forceinline__ TileRows find_tile_wave(int mt, int BM, const int32_t
 
 __device__ __forceinline__ float silu_fast(float g) { return g / (1.0f + __expf(-g)); }
 
+struct TileCoord {
+  int mt, nt;  // mt < 0: this workgroup has no tile
+};
+
+// Workgroup id -> (m-tile, n-tile).  Consecutive workgroup ids go round-robin to the 8 XCDs, so
+// each XCD gets a contiguous range of the logical order, and that order is walked in groups of
+// group_m m-tiles x all n-tiles so that neighbours share operand panels in their L2.
+__device__ __forceinline__ TileCoord xcd_tile_order(int mtiles, int ntiles_n, int group_m) {
+  TileCoord t;
+  const int total = mtiles * ntiles_n;
+  const int per_xcd = (int)gridDim.x >> 3;
+  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (logical >= total) {
+    t.mt = -1;
+    t.nt = 0;
+    return t;
+  }
+  const int group_span = group_m * ntiles_n;
+  const int group = logical / group_span;
+  const int in_group = logical - group * group_span;
+  const int gm = min(group_m, mtiles - group * group_m);
+  t.nt = in_group / gm;
+  t.mt = group * group_m + (in_group - t.nt * gm);
+  return t;
+}
+
+// Second half of every epilogue: a wave has parked its WM x WNO block of bf16 results in its own
+// LDS slice `cw` (row stride CS elements) and streams it out row by row with 16-byte stores.
+// Row r of the block is output row out_row0 + r; rows at or past rows_end and columns at or past
+// N are dropped.
+template <int WM, int WNO, int CS>
+__device__ __forceinline__ void store_wave_block(const uint16_t* __restrict__ cw, int lane, uint16_t* __restrict__ out,
+                                                 int N, size_t out_row0, int rows_end, int col0) {
+  constexpr int CPR_OUT = WNO / 8;
+  constexpr int OUT_CHUNKS = WM * CPR_OUT;
+#pragma unroll
+  for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
+    const int c = lane + j * 64;
+    const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
+    const int col = col0 + ch * 8;
+    if (r < rows_end && col < N) *reinterpret_cast<u32x4_t*>(out + (out_row0 + r) * N + col) = v;
+  }
+}
+
 // number of workgroups for `mtiles x ntiles_n` tiles: a multiple of 8 (one slice per XCD)
 inline int64_t gemm_grid(int64_t mtiles, int64_t ntiles_n) { return (mtiles * ntiles_n + 7) / 8 * 8; }
 

@@ -58,16 +58,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
-  const int total = mtiles * ntiles_n;
-  const int per_xcd = (int)gridDim.x >> 3;
-  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
-  if (logical >= total) return;
-  const int group_span = Cfg::GROUP_M * ntiles_n;
-  const int group = logical / group_span;
-  const int in_group = logical - group * group_span;
-  const int gm = min(Cfg::GROUP_M, mtiles - group * Cfg::GROUP_M);
-  const int nt = in_group / gm;
-  const int mt = group * Cfg::GROUP_M + (in_group - nt * gm);
+  const TileCoord tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
+  if (tc.mt < 0) return;
+  const int mt = tc.mt, nt = tc.nt;
 
   TileRows tr = find_tile_wave(mt, BM, group_sizes, offsets, E, dense_rows);
   tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
@@ -189,19 +182,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
         const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
         cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj][i]);
       }
-  constexpr int CPR_OUT = WN / 8;
-  constexpr int OUT_CHUNKS = WM * CPR_OUT;
-  const int col0 = n0 + wn * WN;
-  const int row_base = wm * WM;
-#pragma unroll
-  for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
-    const int c = lane + j * 64;
-    const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
-    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
-    const int col = col0 + ch * 8;
-    if (row_base + r < tr.rows && col < N)
-      *reinterpret_cast<u32x4_t*>(C + (size_t)(tr.row0 + row_base + r) * N + col) = v;
-  }
+  store_wave_block<WM, WN, CS>(cw, lane, C, N, (size_t)tr.row0 + wm * WM, tr.rows - wm * WM, n0 + wn * WN);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -429,8 +410,6 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   }
   // epilogue: per matrix, each wave parks its WM x WNO block in LDS and streams it out in rows
   uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
-  constexpr int CPR_OUT = WNO / 8;
-  constexpr int OUT_CHUNKS = WM * CPR_OUT;
   const int col0 = n0 + wn * WNO;
   const int row_base = m0 + wm * WM;
 #pragma unroll
@@ -445,14 +424,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
           cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj + which * (TN / 2)][i]);
         }
     uint16_t* const Cm = (which ? C1 : C0) + (size_t)e * KA * N;
-#pragma unroll
-    for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
-      const int c = lane + j * 64;
-      const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
-      const int col = col0 + ch * 8;
-      if (row_base + r < KA && col < N) *reinterpret_cast<u32x4_t*>(Cm + (size_t)(row_base + r) * N + col) = v;
-    }
+    store_wave_block<WM, WNO, CS>(cw, lane, Cm, N, (size_t)row_base, KA - row_base, col0);
     // the staging area is private to the wave and the second matrix is written by the same
     // lanes' LDS stores after their loads above: program order within the wave suffices
   }

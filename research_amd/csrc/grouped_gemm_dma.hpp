@@ -116,19 +116,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   constexpr bool kDual = Cfg::kDual;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
-  // ---- block -> (m-tile, n-tile): consecutive workgroup ids go round-robin to the 8 XCDs,
-  // so give each XCD a contiguous range of the logical order, and walk that order in groups
-  // of GROUP_M m-tiles x all n-tiles so that neighbours share operand panels in their L2.
-  const int total = mtiles * ntiles_n;
-  const int per_xcd = (int)gridDim.x >> 3;
-  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
-  if (logical >= total) return;
-  const int group_span = Cfg::GROUP_M * ntiles_n;
-  const int group = logical / group_span;
-  const int in_group = logical - group * group_span;
-  const int gm = min(Cfg::GROUP_M, mtiles - group * Cfg::GROUP_M);
-  const int nt = in_group / gm;
-  const int mt = group * Cfg::GROUP_M + (in_group - nt * gm);
+  const TileCoord tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
+  if (tc.mt < 0) return;
+  const int mt = tc.mt, nt = tc.nt;
 
   TileRows tr = find_tile_wave(mt, BM, group_sizes, offsets, E, dense_rows);
   tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
@@ -295,8 +285,6 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   // pass needs, are written as well: pass 0 stores the result, passes 1 and 2 the two products.
   constexpr int TNO = Cfg::TNO, WNO = Cfg::WNO, CS = Cfg::CS;
   uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
-  constexpr int CPR_OUT = WNO / 8;
-  constexpr int OUT_CHUNKS = WM * CPR_OUT;
   const int col0 = n0 + wn * WNO;
   const int row_base = wm * WM;
   const int passes = (kDual && save0 != nullptr) ? 3 : 1;
@@ -321,15 +309,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
       }
     }
     uint16_t* const out = pass == 0 ? C : (pass == 1 ? save0 : save1);
-#pragma unroll
-    for (int j = 0; j < OUT_CHUNKS / 64; ++j) {
-      const int c = lane + j * 64;
-      const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
-      const int col = col0 + ch * 8;
-      if (row_base + r < tr.rows && col < N)
-        *reinterpret_cast<u32x4_t*>(out + (size_t)(tr.row0 + row_base + r) * N + col) = v;
-    }
+    store_wave_block<WM, WNO, CS>(cw, lane, out, N, (size_t)tr.row0 + row_base, tr.rows - row_base, col0);
   }
 }
 
