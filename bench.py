@@ -197,7 +197,7 @@ def main() -> int:
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=3)
     parser.add_argument("--config", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
-    parser.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    parser.add_argument("--cpu-sample-tokens", type=int, default=8192)
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-train", action="store_true", help="skip the forward+backward timing")
     parser.add_argument("--no-block", action="store_true", help="skip the decoder-block and graph-replay timings")
