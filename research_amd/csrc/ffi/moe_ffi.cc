@@ -153,6 +153,138 @@ ffi::Error MoeCombine(hipStream_t stream, ffi::AnyBuffer packed_y, ffi::Buffer<f
   return status_to_error(rc);
 }
 
+// Forward that keeps the residuals of the backward pass.  Same operands as MoeForward; four more
+// results: gate_pre, up_pre [A, I] and shared_gate_pre, shared_up_pre [T, Is].
+ffi::Error MoeForwardTrain(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer w_router,
+                           ffi::Buffer<ffi::DataType::F32> expert_bias, ffi::AnyBuffer gate, ffi::AnyBuffer up,
+                           ffi::AnyBuffer down, ffi::AnyBuffer shared_gate, ffi::AnyBuffer shared_up,
+                           ffi::AnyBuffer shared_down, ffi::Result<ffi::AnyBuffer> y,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> expert_ids,
+                           ffi::Result<ffi::AnyBuffer> weights, ffi::Result<ffi::Buffer<ffi::DataType::F32>> scores,
+                           ffi::Result<ffi::Buffer<ffi::DataType::F32>> expert_counts,
+                           ffi::Result<ffi::Buffer<ffi::DataType::F32>> importance,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> group_sizes,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> offsets,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> source_order,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> inverse, ffi::Result<ffi::AnyBuffer> gate_pre,
+                           ffi::Result<ffi::AnyBuffer> up_pre, ffi::Result<ffi::AnyBuffer> shared_gate_pre,
+                           ffi::Result<ffi::AnyBuffer> shared_up_pre,
+                           ffi::Result<ffi::Buffer<ffi::DataType::U8>> workspace, int64_t top_k, double route_scale) {
+  const auto xd = x.dimensions();
+  const auto gd = gate.dimensions();
+  if (xd.size() < 2 || gd.size() != 3) return ffi::Error::InvalidArgument("moe expects x [..., H] and gate [E, H, I]");
+  const int dtype = dtype_code(x.element_type());
+  if (dtype < 0) return ffi::Error::InvalidArgument("moe compute dtype must be bfloat16 or float32");
+  const int64_t H = xd.back(), T = leading(xd), E = gd[0], I = gd[2];
+  const int64_t Is = shared_gate.dimensions().size() == 2 ? shared_gate.dimensions()[1] : 0;
+  if (gd[1] != H) return ffi::Error::InvalidArgument("expert gate matrix must be [E, H, I]");
+  if (workspace->element_count() < jtmoe_workspace_bytes(T, H, E, top_k, I, Is, dtype))
+    return ffi::Error::InvalidArgument("moe workspace result buffer is too small");
+  const int rc = jtmoe_moe_forward_train(
+      x.untyped_data(), w_router.untyped_data(), expert_bias.typed_data(), gate.untyped_data(), up.untyped_data(),
+      down.untyped_data(), Is ? shared_gate.untyped_data() : nullptr, Is ? shared_up.untyped_data() : nullptr,
+      Is ? shared_down.untyped_data() : nullptr, T, H, E, top_k, I, Is, route_scale, dtype, y->untyped_data(),
+      expert_ids->typed_data(), weights->untyped_data(), scores->typed_data(), expert_counts->typed_data(),
+      importance->typed_data(), group_sizes->typed_data(), offsets->typed_data(), source_order->typed_data(),
+      inverse->typed_data(), gate_pre->untyped_data(), up_pre->untyped_data(),
+      Is ? shared_gate_pre->untyped_data() : nullptr, Is ? shared_up_pre->untyped_data() : nullptr,
+      workspace->typed_data(), workspace->element_count(), stream);
+  return status_to_error(rc);
+}
+
+// Vector-Jacobian product of the layer for the cotangents dy [..., H] and d_scores [..., E].
+ffi::Error MoeBackward(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer dy,
+                       ffi::Buffer<ffi::DataType::F32> d_scores, ffi::AnyBuffer w_router, ffi::AnyBuffer gate,
+                       ffi::AnyBuffer up, ffi::AnyBuffer down, ffi::AnyBuffer shared_gate, ffi::AnyBuffer shared_up,
+                       ffi::AnyBuffer shared_down, ffi::Buffer<ffi::DataType::F32> scores,
+                       ffi::Buffer<ffi::DataType::S32> expert_ids, ffi::AnyBuffer weights,
+                       ffi::Buffer<ffi::DataType::S32> source_order, ffi::Buffer<ffi::DataType::S32> inverse,
+                       ffi::Buffer<ffi::DataType::S32> group_sizes, ffi::Buffer<ffi::DataType::S32> offsets,
+                       ffi::AnyBuffer gate_pre, ffi::AnyBuffer up_pre, ffi::AnyBuffer shared_gate_pre,
+                       ffi::AnyBuffer shared_up_pre, ffi::Result<ffi::AnyBuffer> dx,
+                       ffi::Result<ffi::AnyBuffer> d_w_router, ffi::Result<ffi::AnyBuffer> d_gate,
+                       ffi::Result<ffi::AnyBuffer> d_up, ffi::Result<ffi::AnyBuffer> d_down,
+                       ffi::Result<ffi::AnyBuffer> d_shared_gate, ffi::Result<ffi::AnyBuffer> d_shared_up,
+                       ffi::Result<ffi::AnyBuffer> d_shared_down,
+                       ffi::Result<ffi::Buffer<ffi::DataType::U8>> workspace, double route_scale) {
+  const auto xd = x.dimensions();
+  const auto gd = gate.dimensions();
+  const auto id = expert_ids.dimensions();
+  if (xd.size() < 2 || gd.size() != 3 || id.size() < 1)
+    return ffi::Error::InvalidArgument("moe backward expects x [..., H], gate [E, H, I] and ids [..., K]");
+  const int dtype = dtype_code(x.element_type());
+  if (dtype < 0 || dy.element_type() != x.element_type())
+    return ffi::Error::InvalidArgument("moe backward: x and dy must both be bfloat16 or float32");
+  const int64_t H = xd.back(), T = leading(xd), E = gd[0], I = gd[2], K = id.back();
+  const int64_t Is = shared_gate.dimensions().size() == 2 ? shared_gate.dimensions()[1] : 0;
+  if (workspace->element_count() < jtmoe_moe_backward_workspace_bytes(T, H, E, K, I, Is, dtype))
+    return ffi::Error::InvalidArgument("moe backward workspace result buffer is too small");
+  const int rc = jtmoe_moe_backward(
+      x.untyped_data(), dy.untyped_data(), d_scores.typed_data(), w_router.untyped_data(), gate.untyped_data(),
+      up.untyped_data(), down.untyped_data(), Is ? shared_gate.untyped_data() : nullptr,
+      Is ? shared_up.untyped_data() : nullptr, Is ? shared_down.untyped_data() : nullptr, scores.typed_data(),
+      expert_ids.typed_data(), weights.untyped_data(), source_order.typed_data(), inverse.typed_data(),
+      group_sizes.typed_data(), offsets.typed_data(), gate_pre.untyped_data(), up_pre.untyped_data(),
+      Is ? shared_gate_pre.untyped_data() : nullptr, Is ? shared_up_pre.untyped_data() : nullptr, route_scale, T, H,
+      E, K, I, Is, dtype, dx->untyped_data(), d_w_router->untyped_data(), d_gate->untyped_data(),
+      d_up->untyped_data(), d_down->untyped_data(), Is ? d_shared_gate->untyped_data() : nullptr,
+      Is ? d_shared_up->untyped_data() : nullptr, Is ? d_shared_down->untyped_data() : nullptr,
+      workspace->typed_data(), workspace->element_count(), stream);
+  return status_to_error(rc);
+}
+
+// RMSNorm with a float32 scale, the operands of the reference's own handler
+// (rmsnorm_ffi.cu:24-74) for any hidden size and both dtypes.
+ffi::Error Rmsnorm(hipStream_t stream, ffi::AnyBuffer x, ffi::Buffer<ffi::DataType::F32> scale,
+                   ffi::Result<ffi::AnyBuffer> y, double eps) {
+  const auto xd = x.dimensions();
+  if (xd.size() < 2) return ffi::Error::InvalidArgument("rmsnorm input rank must be at least 2");
+  if (scale.element_count() != static_cast<size_t>(xd.back()))
+    return ffi::Error::InvalidArgument("rmsnorm scale must have shape [H]");
+  const int dtype = dtype_code(x.element_type());
+  if (dtype < 0) return ffi::Error::InvalidArgument("rmsnorm dtype must be bfloat16 or float32");
+  return status_to_error(
+      jtmoe_rmsnorm(x.untyped_data(), scale.typed_data(), leading(xd), xd.back(), eps, dtype, y->untyped_data(), stream));
+}
+
+// x + post_norm(moe(pre_norm(x))): operands of MoeForward preceded by x's two norm scales.
+ffi::Error FfnBlockForward(hipStream_t stream, ffi::AnyBuffer x, ffi::Buffer<ffi::DataType::F32> pre_scale,
+                           ffi::Buffer<ffi::DataType::F32> post_scale, ffi::AnyBuffer w_router,
+                           ffi::Buffer<ffi::DataType::F32> expert_bias, ffi::AnyBuffer gate, ffi::AnyBuffer up,
+                           ffi::AnyBuffer down, ffi::AnyBuffer shared_gate, ffi::AnyBuffer shared_up,
+                           ffi::AnyBuffer shared_down, ffi::Result<ffi::AnyBuffer> out,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> expert_ids,
+                           ffi::Result<ffi::AnyBuffer> weights, ffi::Result<ffi::Buffer<ffi::DataType::F32>> scores,
+                           ffi::Result<ffi::Buffer<ffi::DataType::F32>> expert_counts,
+                           ffi::Result<ffi::Buffer<ffi::DataType::F32>> importance,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> group_sizes,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> offsets,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> source_order,
+                           ffi::Result<ffi::Buffer<ffi::DataType::S32>> inverse,
+                           ffi::Result<ffi::Buffer<ffi::DataType::U8>> workspace, int64_t top_k, double route_scale,
+                           double eps) {
+  const auto xd = x.dimensions();
+  const auto gd = gate.dimensions();
+  if (xd.size() < 2 || gd.size() != 3) return ffi::Error::InvalidArgument("block expects x [..., H] and gate [E, H, I]");
+  const int dtype = dtype_code(x.element_type());
+  if (dtype < 0) return ffi::Error::InvalidArgument("block compute dtype must be bfloat16 or float32");
+  const int64_t H = xd.back(), T = leading(xd), E = gd[0], I = gd[2];
+  const int64_t Is = shared_gate.dimensions().size() == 2 ? shared_gate.dimensions()[1] : 0;
+  if (pre_scale.element_count() != static_cast<size_t>(H) || post_scale.element_count() != static_cast<size_t>(H))
+    return ffi::Error::InvalidArgument("norm scales must have shape [H]");
+  if (workspace->element_count() < jtmoe_ffn_block_workspace_bytes(T, H, E, top_k, I, Is, dtype))
+    return ffi::Error::InvalidArgument("block workspace result buffer is too small");
+  const int rc = jtmoe_ffn_block_forward(
+      x.untyped_data(), pre_scale.typed_data(), post_scale.typed_data(), eps, w_router.untyped_data(),
+      expert_bias.typed_data(), gate.untyped_data(), up.untyped_data(), down.untyped_data(),
+      Is ? shared_gate.untyped_data() : nullptr, Is ? shared_up.untyped_data() : nullptr,
+      Is ? shared_down.untyped_data() : nullptr, T, H, E, top_k, I, Is, route_scale, dtype, out->untyped_data(),
+      expert_ids->typed_data(), weights->untyped_data(), scores->typed_data(), expert_counts->typed_data(),
+      importance->typed_data(), group_sizes->typed_data(), offsets->typed_data(), source_order->typed_data(),
+      inverse->typed_data(), workspace->typed_data(), workspace->element_count(), stream);
+  return status_to_error(rc);
+}
+
 }  // namespace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanMoeForward, MoeForward,
@@ -227,3 +359,58 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanMoeCombine, MoeCombine,
                                   .Arg<ffi::Buffer<ffi::DataType::S32>>()
                                   .Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>());
+
+#define JT_ANY .Arg<ffi::AnyBuffer>()
+#define JT_F32 .Arg<ffi::Buffer<ffi::DataType::F32>>()
+#define JT_S32 .Arg<ffi::Buffer<ffi::DataType::S32>>()
+#define JT_RANY .Ret<ffi::AnyBuffer>()
+#define JT_RF32 .Ret<ffi::Buffer<ffi::DataType::F32>>()
+#define JT_RS32 .Ret<ffi::Buffer<ffi::DataType::S32>>()
+#define JT_RU8 .Ret<ffi::Buffer<ffi::DataType::U8>>()
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanMoeForwardTrain, MoeForwardTrain,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  JT_ANY JT_ANY JT_F32 JT_ANY JT_ANY JT_ANY JT_ANY JT_ANY JT_ANY  // as MoeForward
+                                  JT_RANY JT_RS32 JT_RANY JT_RF32 JT_RF32 JT_RF32 JT_RS32 JT_RS32 JT_RS32 JT_RS32
+                                  JT_RANY JT_RANY JT_RANY JT_RANY  // gate_pre, up_pre, shared_gate_pre, shared_up_pre
+                                  JT_RU8
+                                  .Attr<int64_t>("top_k")
+                                  .Attr<double>("route_scale"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanMoeBackward, MoeBackward,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  JT_ANY JT_ANY JT_F32                             // x, dy, d_scores
+                                  JT_ANY JT_ANY JT_ANY JT_ANY JT_ANY JT_ANY JT_ANY  // router, gate, up, down, shared x3
+                                  JT_F32 JT_S32 JT_ANY                             // scores, expert_ids, weights
+                                  JT_S32 JT_S32 JT_S32 JT_S32                      // source_order, inverse, sizes, offsets
+                                  JT_ANY JT_ANY JT_ANY JT_ANY                      // the four residuals
+                                  JT_RANY JT_RANY JT_RANY JT_RANY JT_RANY JT_RANY JT_RANY JT_RANY  // the eight gradients
+                                  JT_RU8
+                                  .Attr<double>("route_scale"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanRmsnorm, Rmsnorm,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  JT_ANY JT_F32 JT_RANY
+                                  .Attr<double>("eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanFfnBlockForward, FfnBlockForward,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  JT_ANY JT_F32 JT_F32                                              // x, pre, post scale
+                                  JT_ANY JT_F32 JT_ANY JT_ANY JT_ANY JT_ANY JT_ANY JT_ANY            // as MoeForward after x
+                                  JT_RANY JT_RS32 JT_RANY JT_RF32 JT_RF32 JT_RF32 JT_RS32 JT_RS32 JT_RS32 JT_RS32
+                                  JT_RU8
+                                  .Attr<int64_t>("top_k")
+                                  .Attr<double>("route_scale")
+                                  .Attr<double>("eps"));
+
+#undef JT_ANY
+#undef JT_F32
+#undef JT_S32
+#undef JT_RANY
+#undef JT_RF32
+#undef JT_RS32
+#undef JT_RU8

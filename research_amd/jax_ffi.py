@@ -24,6 +24,10 @@ TARGETS = {
     "jaxtitan_moe_dispatch": "JaxtitanMoeDispatch",
     "jaxtitan_moe_grouped_swiglu": "JaxtitanMoeGroupedSwiglu",
     "jaxtitan_moe_combine": "JaxtitanMoeCombine",
+    "jaxtitan_moe_forward_train": "JaxtitanMoeForwardTrain",
+    "jaxtitan_moe_backward": "JaxtitanMoeBackward",
+    "jaxtitan_rmsnorm": "JaxtitanRmsnorm",
+    "jaxtitan_ffn_block_forward": "JaxtitanFfnBlockForward",
 }
 
 _REGISTERED: set[str] = set()
@@ -97,3 +101,80 @@ def moe_forward(x: Any, router_kernel: Any, expert_bias: Any, gate: Any, up: Any
     out = call(x, router_kernel, expert_bias, gate, up, down, *shared, top_k=int(top_k),
                route_scale=float(route_scale))
     return out[:6]
+
+
+def moe_layer(x: Any, router_kernel: Any, expert_bias: Any, gate: Any, up: Any, down: Any, *, top_k: int,
+              route_scale: float = 1.0, shared: tuple[Any, Any, Any] | None = None,
+              cache_root: str | Path | None = None):
+    """The layer with its custom VJP (docs/kernel_backend_design.md:120-128 of the reference):
+    returns (y, scores, expert_ids); differentiable in x, the router kernel, the expert matrices and
+    the shared-expert matrices, with cotangents on y and on the scores."""
+    jax = _jax()
+    import jax.numpy as jnp  # noqa: PLC0415
+
+    register_moe(cache_root)
+    from research_amd import _ffi  # noqa: PLC0415
+
+    lead, hidden = x.shape[:-1], x.shape[-1]
+    tokens = 1
+    for n in lead:
+        tokens *= n
+    experts, _, inter = gate.shape
+    if shared is None:
+        shared = (jnp.zeros((hidden, 0), x.dtype), jnp.zeros((hidden, 0), x.dtype), jnp.zeros((0, hidden), x.dtype))
+    shared_inter = shared[0].shape[1]
+    code = _ffi.JTMOE_BF16 if x.dtype == jnp.bfloat16 else _ffi.JTMOE_F32
+    lib = _ffi.load_library(cache_root)
+    fwd_ws = max(int(lib.jtmoe_workspace_bytes(tokens, hidden, experts, top_k, inter, shared_inter, code)), 256)
+    bwd_ws = max(int(lib.jtmoe_moe_backward_workspace_bytes(tokens, hidden, experts, top_k, inter, shared_inter,
+                                                            code)), 256)
+    sds = jax.ShapeDtypeStruct
+    rows = tokens * top_k
+    i32, f32 = jnp.int32, jnp.float32
+
+    def forward_call(x, router_kernel, gate, up, down, shared):
+        out = jax.ffi.ffi_call(
+            "jaxtitan_moe_forward_train",
+            (
+                sds(x.shape, x.dtype), sds((*lead, top_k), i32), sds((*lead, top_k), x.dtype),
+                sds((*lead, experts), f32), sds((experts,), f32), sds((experts,), f32), sds((experts,), i32),
+                sds((experts,), i32), sds((rows,), i32), sds((rows,), i32),
+                sds((rows, inter), x.dtype), sds((rows, inter), x.dtype),
+                sds((tokens, shared_inter), x.dtype), sds((tokens, shared_inter), x.dtype),
+                sds((fwd_ws,), jnp.uint8),
+            ),
+            vmap_method="sequential",
+        )(x, router_kernel, jax.lax.stop_gradient(expert_bias), gate, up, down, *shared, top_k=int(top_k),
+          route_scale=float(route_scale))
+        return out[:-1]
+
+    @jax.custom_vjp
+    def layer(x, router_kernel, gate, up, down, shared):
+        y, ids, _, scores = forward_call(x, router_kernel, gate, up, down, shared)[:4]
+        return y, scores, ids
+
+    def layer_fwd(x, router_kernel, gate, up, down, shared):
+        out = forward_call(x, router_kernel, gate, up, down, shared)
+        y, ids, weights, scores = out[:4]
+        plan, residuals = out[6:10], out[10:14]
+        return (y, scores, ids), (x, router_kernel, gate, up, down, shared, scores, ids, weights, plan, residuals)
+
+    def layer_bwd(saved, cotangents):
+        x, router_kernel, gate, up, down, shared, scores, ids, weights, plan, residuals = saved
+        dy, d_scores, _ = cotangents
+        group_sizes, offsets, source_order, inverse = plan
+        grads = jax.ffi.ffi_call(
+            "jaxtitan_moe_backward",
+            (
+                sds(x.shape, x.dtype), sds(router_kernel.shape, x.dtype), sds(gate.shape, x.dtype),
+                sds(up.shape, x.dtype), sds(down.shape, x.dtype), sds(shared[0].shape, x.dtype),
+                sds(shared[1].shape, x.dtype), sds(shared[2].shape, x.dtype), sds((bwd_ws,), jnp.uint8),
+            ),
+            vmap_method="sequential",
+        )(x, dy, d_scores.astype(f32), router_kernel, gate, up, down, *shared, scores, ids, weights, source_order,
+          inverse, group_sizes, offsets, *residuals, route_scale=float(route_scale))
+        dx, d_router, d_gate, d_up, d_down, dsg, dsu, dsd = grads[:8]
+        return dx, d_router, d_gate, d_up, d_down, (dsg, dsu, dsd)
+
+    layer.defvjp(layer_fwd, layer_bwd)
+    return layer(x, router_kernel, gate, up, down, shared)
