@@ -73,7 +73,10 @@ def test_jax_ffi_stub_fails_loudly_without_jax():
         jax_ffi.register_moe()
     assert set(jax_ffi.TARGETS.values()) == {
         "JaxtitanMoeForward", "JaxtitanMoeRouter", "JaxtitanMoeDispatch", "JaxtitanMoeGroupedSwiglu",
-        "JaxtitanMoeCombine"}
+        "JaxtitanMoeCombine", "JaxtitanMoeForwardTrain", "JaxtitanMoeBackward", "JaxtitanRmsnorm",
+        "JaxtitanFfnBlockForward"}
+    with pytest.raises(ContractError, match="jax is not installed"):
+        jax_ffi.moe_layer(None, None, None, None, None, None, top_k=1)
 
 
 def test_training_and_block_operators_refuse_cpu_tensors_and_bad_shapes():
