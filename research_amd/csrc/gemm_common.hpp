@@ -21,32 +21,27 @@ struct TileRows {
   int rows;  // valid rows in the tile (0 = no such tile)
 };
 
-// m-tile `mt` counted expert by expert (ceil(group_size / BM) tiles each).  Every
-// lane of the calling wave gets the same answer.  E <= 256.
-__device__ __forceinline__ TileRows find_tile_wave(int mt, int BM, const int32_t* __restrict__ group_sizes,
-                                                   const int32_t* __restrict__ offsets, int E, int dense_rows) {
-  TileRows r;
-  r.expert = 0;
-  r.row0 = 0;
-  r.rows = 0;
-  if (group_sizes == nullptr) {
-    const int row0 = mt * BM;
-    if (row0 < dense_rows) {
-      r.row0 = row0;
-      r.rows = min(BM, dense_rows - row0);
-    }
-    return r;
-  }
-  const int lane = threadIdx.x & 63;
-  constexpr int kPer = JTMOE_MAX_EXPERTS / 64;  // experts per lane, contiguous
+// Tiles are counted expert by expert, ceil(group_size / BM) m-tiles each.  group_scan computes, in
+// every lane of the calling wave, the tile counts of the lane's own experts, their exclusive
+// prefix and the total; locate_tile then finds the expert and row range of m-tile `mt`.
+// E <= JTMOE_MAX_EXPERTS.
+struct GroupScan {
+  static constexpr int kPer = JTMOE_MAX_EXPERTS / 64;  // experts per lane, contiguous
   int n[kPer], tiles[kPer];
+  int first;  // tiles before this lane's experts
+  int total;  // tiles of all experts
+};
+
+__device__ __forceinline__ GroupScan group_scan(int BM, const int32_t* __restrict__ group_sizes, int E) {
+  GroupScan g;
+  const int lane = threadIdx.x & 63;
   int local = 0;
 #pragma unroll
-  for (int j = 0; j < kPer; ++j) {
-    const int e = lane * kPer + j;
-    n[j] = e < E ? group_sizes[e] : 0;
-    tiles[j] = (n[j] + BM - 1) / BM;
-    local += tiles[j];
+  for (int j = 0; j < GroupScan::kPer; ++j) {
+    const int e = lane * GroupScan::kPer + j;
+    g.n[j] = e < E ? group_sizes[e] : 0;
+    g.tiles[j] = (g.n[j] + BM - 1) / BM;
+    local += g.tiles[j];
   }
   int incl = local;
 #pragma unroll
@@ -54,20 +49,35 @@ __device__ __forceinline__ TileRows find_tile_wave(int mt, int BM, const int32_t
     const int v = __shfl_up(incl, d);
     if (lane >= d) incl += v;
   }
-  int first = incl - local;  // tiles before this lane's experts
-  const bool mine = mt >= first && mt < incl;
+  g.first = incl - local;
+  g.total = __shfl(incl, 63);
+  return g;
+}
+
+__device__ __forceinline__ TileRows locate_tile(const GroupScan& g, int mt, int BM,
+                                                const int32_t* __restrict__ offsets) {
+  TileRows r;
+  r.expert = 0;
+  r.row0 = 0;
+  r.rows = 0;
+  const int lane = threadIdx.x & 63;
+  int first = g.first;
+  int last = first;
+#pragma unroll
+  for (int j = 0; j < GroupScan::kPer; ++j) last += g.tiles[j];
+  const bool mine = mt >= first && mt < last;
   const unsigned long long owners = __ballot(mine);
   if (owners == 0ull) return r;
   const int owner = __ffsll((long long)owners) - 1;
   int expert = 0, local_tile = 0, rows_e = 0;
 #pragma unroll
-  for (int j = 0; j < kPer; ++j) {
-    if (mine && mt >= first && mt < first + tiles[j]) {
-      expert = lane * kPer + j;
+  for (int j = 0; j < GroupScan::kPer; ++j) {
+    if (mine && mt >= first && mt < first + g.tiles[j]) {
+      expert = lane * GroupScan::kPer + j;
       local_tile = mt - first;
-      rows_e = n[j];
+      rows_e = g.n[j];
     }
-    first += tiles[j];
+    first += g.tiles[j];
   }
   expert = __shfl(expert, owner);
   local_tile = __shfl(local_tile, owner);
@@ -76,6 +86,25 @@ __device__ __forceinline__ TileRows find_tile_wave(int mt, int BM, const int32_t
   r.row0 = offsets[expert] + local_tile * BM;
   r.rows = min(BM, rows_e - local_tile * BM);
   return r;
+}
+
+// m-tile `mt` of a grouped (or, with group_sizes == nullptr, dense) row range.  Every lane of the
+// calling wave gets the same answer.
+__device__ __forceinline__ TileRows find_tile_wave(int mt, int BM, const int32_t* __restrict__ group_sizes,
+                                                   const int32_t* __restrict__ offsets, int E, int dense_rows) {
+  if (group_sizes == nullptr) {
+    TileRows r;
+    r.expert = 0;
+    r.row0 = 0;
+    r.rows = 0;
+    const int row0 = mt * BM;
+    if (row0 < dense_rows) {
+      r.row0 = row0;
+      r.rows = min(BM, dense_rows - row0);
+    }
+    return r;
+  }
+  return locate_tile(group_scan(BM, group_sizes, E), mt, BM, offsets);
 }
 
 __device__ __forceinline__ float silu_fast(float g) { return g / (1.0f + __expf(-g)); }
@@ -97,6 +126,28 @@ __device__ __forceinline__ TileCoord xcd_tile_order(int mtiles, int ntiles_n, in
     t.nt = 0;
     return t;
   }
+  const int group_span = group_m * ntiles_n;
+  const int group = logical / group_span;
+  const int in_group = logical - group * group_span;
+  const int gm = min(group_m, mtiles - group * group_m);
+  t.nt = in_group / gm;
+  t.mt = group * group_m + (in_group - t.nt * gm);
+  return t;
+}
+
+// The tile of this workgroup when the launch was sized for an upper bound of `mtiles_bound` m-tiles
+// and only `mtiles` of them exist (group sizes live on the device): the XCD ranges are cut from the
+// real count, so that the surplus workgroups are spread over all XCDs instead of idling one of them.
+// Requires gridDim.x / 8 >= ceil(mtiles * ntiles_n / 8), which the bound guarantees.
+__device__ __forceinline__ TileCoord xcd_tile_order_balanced(int mtiles, int ntiles_n, int group_m) {
+  TileCoord t;
+  t.mt = -1;
+  t.nt = 0;
+  const int total = mtiles * ntiles_n;
+  const int per_xcd = (total + 7) >> 3;
+  const int idx = (int)blockIdx.x >> 3;
+  const int logical = ((int)blockIdx.x & 7) * per_xcd + idx;
+  if (idx >= per_xcd || logical >= total) return t;
   const int group_span = group_m * ntiles_n;
   const int group = logical / group_span;
   const int in_group = logical - group * group_span;

@@ -58,11 +58,20 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
-  const TileCoord tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
-  if (tc.mt < 0) return;
-  const int mt = tc.mt, nt = tc.nt;
-
-  TileRows tr = find_tile_wave(mt, BM, group_sizes, offsets, E, dense_rows);
+  // the grid covers an upper bound of the m-tiles; the tile order is cut from their real number
+  TileCoord tc;
+  TileRows tr;
+  if (group_sizes) {
+    const GroupScan scan = group_scan(BM, group_sizes, E);
+    tc = xcd_tile_order_balanced(scan.total, ntiles_n, Cfg::GROUP_M);
+    if (tc.mt < 0) return;
+    tr = locate_tile(scan, tc.mt, BM, offsets);
+  } else {
+    tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
+    if (tc.mt < 0) return;
+    tr = find_tile_wave(tc.mt, BM, nullptr, nullptr, E, dense_rows);
+  }
+  const int nt = tc.nt;
   tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
   tr.row0 = __builtin_amdgcn_readfirstlane(tr.row0);
   tr.rows = __builtin_amdgcn_readfirstlane(tr.rows);
@@ -141,11 +150,14 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
       bf[jj] = *reinterpret_cast<const bf16x8_t*>(st + b_rowoff + jj * 32 * BK * 2 + chunk);
   };
 
+  // a wave whose rows all lie past the end of the group skips its fragment reads and MFMAs
+  const bool wave_has_rows = wm * WM < tr.rows;
   if (nk > 0) issue(0);
   for (int kt = 0; kt < nk; ++kt) {
     wait_vmcnt<0>();
     __syncthreads();
     if (kt + 1 < nk) issue(kt + 1);
+    if (!wave_has_rows) continue;
     const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
     bf16x8_t af[2][TM], bf[2][TN];
     load_frags(st, 0, af[0], bf[0]);

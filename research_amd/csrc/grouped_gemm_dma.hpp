@@ -116,11 +116,20 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   constexpr bool kDual = Cfg::kDual;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
-  const TileCoord tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
-  if (tc.mt < 0) return;
-  const int mt = tc.mt, nt = tc.nt;
-
-  TileRows tr = find_tile_wave(mt, BM, group_sizes, offsets, E, dense_rows);
+  // the grid covers an upper bound of the m-tiles; the tile order is cut from their real number
+  TileCoord tc;
+  TileRows tr;
+  if (group_sizes) {
+    const GroupScan scan = group_scan(BM, group_sizes, E);
+    tc = xcd_tile_order_balanced(scan.total, ntiles_n, Cfg::GROUP_M);
+    if (tc.mt < 0) return;
+    tr = locate_tile(scan, tc.mt, BM, offsets);
+  } else {
+    tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
+    if (tc.mt < 0) return;
+    tr = find_tile_wave(tc.mt, BM, nullptr, nullptr, E, dense_rows);
+  }
+  const int nt = tc.nt;
   tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
   tr.row0 = __builtin_amdgcn_readfirstlane(tr.row0);
   tr.rows = __builtin_amdgcn_readfirstlane(tr.rows);
@@ -226,6 +235,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   };
 
   const int nk = Kdim / BK;
+  // The last tile of a group is usually partly empty.  A wave whose WM rows all lie past the end of
+  // the group still takes part in the loads and the barriers but skips its fragment reads and MFMAs.
+  const bool wave_has_rows = wm * WM < tr.rows;
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s)
     if (s < nk) issue(s);
@@ -238,6 +250,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     __syncthreads();
     if (kt + NSTAGE - 1 < nk) issue(kt + NSTAGE - 1);
     const unsigned char* st = smem_raw + (kt % NSTAGE) * Cfg::STAGE_BYTES;
+    if (!wave_has_rows) continue;  // a tile at the end of a group: this wave's rows lie past it
     if (Cfg::OPT & 16) {
       // fragments of step kk+1 are requested before the MFMAs of step kk are issued
       bf16x8_t af[2][TM], bf[2][TN];
