@@ -73,7 +73,7 @@ def test_rmsnorm_reference_known_answer_and_contract(gpu):
 
 @pytest.mark.parametrize("tokens,hidden,top_k,dtype,with_shared",
                          [(300, 2048, 8, "bf16", True), (129, 1024, 2, "bf16", False), (77, 72, 3, "bf16", True),
-                          (50, 40, 2, "f32", True), (64, 4096, 8, "bf16", False)])
+                          (50, 40, 2, "f32", True), (64, 4096, 8, "bf16", False), (33, 8192, 2, "bf16", True)])
 def test_fused_combine_norm_residual(gpu, tokens, hidden, top_k, dtype, with_shared):
     rng = np.random.default_rng(tokens)
     rows = tokens * top_k
