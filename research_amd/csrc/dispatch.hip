@@ -47,24 +47,29 @@ constexpr int kScanThreads = 1024;
 __global__ __launch_bounds__(kScanThreads) void dispatch_scan_kernel(int* __restrict__ partial, int E, int nchunks,
                                                                      int32_t* __restrict__ group_sizes,
                                                                      int32_t* __restrict__ offsets) {
-  __shared__ int sums[kScanThreads];
+  __shared__ int wave_sums[kScanThreads / kWave];
   __shared__ int total_s;
   const int n = E * nchunks;
   const int per = (n + kScanThreads - 1) / kScanThreads;
   const int lo = min(n, (int)threadIdx.x * per), hi = min(n, lo + per);
   int local = 0;
   for (int i = lo; i < hi; ++i) local += partial[i];
-  sums[threadIdx.x] = local;
-  __syncthreads();
-  // Hillis-Steele inclusive scan over the 1024 thread sums
-  for (int d = 1; d < kScanThreads; d <<= 1) {
-    const int v = (int)threadIdx.x >= d ? sums[threadIdx.x - d] : 0;
-    __syncthreads();
-    sums[threadIdx.x] += v;
-    __syncthreads();
+  // inclusive scan of the 1024 thread sums: inside each wave with shuffles, then over the 16 wave
+  // totals (by every wave for itself), two barriers in all
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int incl = local;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int v = __shfl_up(incl, d);
+    if (lane >= d) incl += v;
   }
-  int run = sums[threadIdx.x] - local;
-  if (threadIdx.x == kScanThreads - 1) total_s = sums[threadIdx.x];
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  int before = 0;
+  for (int w = 0; w < wave; ++w) before += wave_sums[w];
+  incl += before;
+  int run = incl - local;
+  if (threadIdx.x == kScanThreads - 1) total_s = incl;
   for (int i = lo; i < hi; ++i) {
     const int v = partial[i];
     partial[i] = run;
