@@ -71,6 +71,49 @@ def test_argument_errors_return_status_and_message_without_a_gpu():
     assert rc == -1 and "workspace" in _ffi.last_error(lib)
 
 
+def test_training_and_block_entry_points_validate_before_launching():
+    lib = _ffi.load_library()
+    bf = _ffi.JTMOE_BF16
+    T, H, E, K, I, Is = 16384, 2048, 64, 8, 1408, 2816
+    b = 2
+    # workspace sizes: pure host arithmetic, at least the buffers they are documented to hold
+    experts = lib.jtmoe_experts_backward_workspace_bytes(T, K, H, I, bf)
+    assert experts >= b * (3 * T * K * I + T * K * H + T * K) and experts % 256 == 0
+    shared = lib.jtmoe_shared_backward_workspace_bytes(T, H, Is, bf)
+    assert shared >= b * 3 * T * Is
+    router = lib.jtmoe_router_backward_workspace_bytes(T, H, E, bf)
+    assert router >= b * T * E
+    whole = lib.jtmoe_moe_backward_workspace_bytes(T, H, E, K, I, Is, bf)
+    assert whole >= experts + shared + router
+    assert lib.jtmoe_moe_backward_workspace_bytes(T, H, E, K, I, Is, 9) == 0
+    assert lib.jtmoe_ffn_block_workspace_bytes(T, H, E, K, I, Is, bf) == \
+        lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, bf) + b * T * H
+    # argument errors come back as a status and a message; nothing is launched
+    rc = lib.jtmoe_rmsnorm(None, None, 4, 8, 1e-6, 9, None, None)
+    assert rc == -1 and "dtype" in _ffi.last_error(lib)
+    rc = lib.jtmoe_rmsnorm(None, None, 4, 8, -1.0, bf, None, None)
+    assert rc == -1 and "eps" in _ffi.last_error(lib)
+    rc = lib.jtmoe_rmsnorm(None, None, 4, 8, 1e-6, bf, None, None)
+    assert rc == -1 and "null" in _ffi.last_error(lib)
+    rc = lib.jtmoe_combine_norm_residual(*([None] * 6), 1e-6, 4, 8, 2, bf, None, None)
+    assert rc == -1 and "null" in _ffi.last_error(lib)
+    rc = lib.jtmoe_experts_backward(*([None] * 12), 4, 2, 8, 8, 300, bf, *([None] * 6), None, 0, None)
+    assert rc == -2 and "exceeds" in _ffi.last_error(lib)
+    rc = lib.jtmoe_experts_backward(*([None] * 12), 4, 2, 8, 8, 4, bf, *([None] * 6), None, 0, None)
+    assert rc == -1 and "null" in _ffi.last_error(lib)
+    rc = lib.jtmoe_shared_backward(*([None] * 7), 4, 8, 8, 9, *([None] * 4), None, 0, None)
+    assert rc == -1 and "dtype" in _ffi.last_error(lib)
+    rc = lib.jtmoe_router_backward(*([None] * 6), 1.0, 4, 8, 4, 17, bf, None, None, None, 0, None)
+    assert rc == -2 and "exceeds" in _ffi.last_error(lib)
+    rc = lib.jtmoe_moe_backward(*([None] * 21), 1.0, 4, 8, 4, 2, 8, 0, bf, *([None] * 8), None, 0, None)
+    assert rc == -1 and "null" in _ffi.last_error(lib)
+    rc = lib.jtmoe_ffn_block_forward(None, None, None, 1e-6, *([None] * 8), 4, 8, 4, 2, 8, 0, 1.0, bf, *([None] * 10),
+                                     None, 0, None)
+    assert rc == -1 and "norm scale" in _ffi.last_error(lib)
+    rc = lib.jtmoe_moe_forward_train(*([None] * 9), 4, 8, 4, 2, 8, 0, 1.0, bf, *([None] * 14), None, 0, None)
+    assert rc == -1 and "residual" in _ffi.last_error(lib)
+
+
 def test_loader_refuses_missing_or_stale_artifacts(tmp_path):
     with pytest.raises(ContractError, match="manifest is missing"):
         _ffi.shared_object_path(tmp_path)
