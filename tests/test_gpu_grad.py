@@ -94,7 +94,7 @@ def test_expert_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, inte
 
 # the 4096-token cases take the path that splits a long one-group reduction into partial sums
 @pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16"),
-                                                       (4096, 512, 704, "bf16")])
+                                                       (4096, 512, 704, "bf16"), (64, 1024, 704, "bf16")])
 def test_shared_gradients_match_oracle(gpu, tokens, hidden, inter, dtype):
     rng = np.random.default_rng(7)
     std = 0.02 if hidden >= 512 else 0.2

@@ -311,7 +311,8 @@ def test_combine_is_bit_exact(gpu, tokens, hidden, top_k, dtype, with_shared):
     assert np.array_equal(host(got), want)
 
 
-@pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16")])
+@pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16"),
+                                                       (64, 1024, 704, "bf16")])
 def test_shared_swiglu_matches_oracle(gpu, tokens, hidden, inter, dtype):
     rng = np.random.default_rng(inter)
     x = rng.standard_normal((tokens, hidden)).astype(np.float32)
