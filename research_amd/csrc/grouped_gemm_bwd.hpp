@@ -287,7 +287,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   const int b_blk_id = kWide ? tid >> 5 : tid >> 3;
   // row inside the k step (first load) and 16-byte chunk inside the 128 columns
   const int l_r = kWide ? (b_blk_id >> 1) * 4 + ((tid >> 3) & 3) : (b_blk_id >> 3) * 4 + ((tid >> 1) & 3);
-  const int l_c = kWide ? (b_blk_id & 1) * 8 + (tid & 7) : (b_blk_id & 7) * 2 + (tid & 1);
+  // (wide blocks: rows 2 and 3 of a block hold their eight chunks with the two halves swapped, which
+  // puts the four 32-byte pieces of a transposing read into four different groups of banks)
+  const int l_c = kWide ? (b_blk_id & 1) * 8 + ((tid & 7) ^ (((tid >> 4) & 1) << 2)) : (b_blk_id & 7) * 2 + (tid & 1);
   constexpr int ROWS_PER_LOAD = NT / 16;
   const int p_col = (m0 + l_c * 8) * 2, d_col = (n0 + l_c * 8) * 2;  // byte offset inside a row
   const unsigned lds0 = lds_byte_addr(smem_raw);
@@ -346,9 +348,12 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
     return kWide ? (col >> 7) * Cfg::SUB_BYTES + ((col & 127) >> 6) * 512 + (col & 63) * 2
                  : (col >> 7) * Cfg::SUB_BYTES + ((col & 127) >> 4) * 128;
   };
+  // the swap of the two 64-byte halves in rows 2 and 3 of a wide block, seen from the reading lane
+  const int half_swap = kWide ? ((lane >> 3) & 1) * 64 : 0;
+  auto swapped = [&](int col) { return (col & 32) ? -half_swap : half_swap; };
   int p_blk[TM], d_blk[TN];
 #pragma unroll
-  for (int mi = 0; mi < TM; ++mi) p_blk[mi] = block_of(wm * WM + mi * 32);
+  for (int mi = 0; mi < TM; ++mi) p_blk[mi] = block_of(wm * WM + mi * 32) + swapped(mi * 32);
 #pragma unroll
   for (int jj = 0; jj < TN; ++jj) {
     int col;
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
       col = (jj < TN / 2 ? 0 : BNO) + wn * (WN / 2) + (jj % (TN / 2)) * 32;
     else
       col = wn * WN + jj * 32;
-    d_blk[jj] = Cfg::P_BYTES + block_of(col);
+    d_blk[jj] = Cfg::P_BYTES + block_of(col) + swapped(col);
   }
   auto read_tr = [&](const unsigned char* p) {
     const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
