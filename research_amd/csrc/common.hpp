@@ -86,4 +86,8 @@ struct Elem<bf16_raw> {
 
 constexpr int kWave = 64;
 
+// dispatch.hip: packed[inverse[t*K + s]] = x[t] (the row scatter of jtmoe_dispatch on its own)
+void launch_dispatch_rows(const void* x, const int32_t* inverse, int64_t T, int64_t K, int64_t H, int dtype,
+                          void* packed_x, hipStream_t stream);
+
 }  // namespace jtmoe

@@ -172,6 +172,36 @@ __global__ __launch_bounds__(256) void dispatch_rows_kernel(const V* __restrict_
 }
 
 }  // namespace
+
+// packed[inverse[t*K + s]] = x[t] for every token t and slot s (rows of H elements)
+void launch_dispatch_rows(const void* x, const int32_t* inverse, int64_t T, int64_t K, int64_t H, int dtype,
+                          void* packed_x, hipStream_t s) {
+  if (T == 0) return;
+  const int64_t A = T * K;
+  const size_t row_bytes = (size_t)H * dtype_bytes(dtype);
+  const bool vec16 = row_bytes % 16 == 0 && aligned16(x) && aligned16(packed_x);
+  if (vec16) {
+    const int row_vecs = (int)(row_bytes / 16);
+    // one wave per row for short rows, up to 256 lanes for long ones
+    int bx = 64;
+    while (bx < 256 && bx * 4 < row_vecs) bx *= 2;
+    dim3 block(bx, 256 / bx);
+    const int grid = (int)((T + block.y - 1) / block.y);
+    dispatch_rows_kernel<uint4><<<grid, block, 0, s>>>(static_cast<const uint4*>(x), inverse, (int)T, (int)K, (int)A,
+                                                       row_vecs, static_cast<uint4*>(packed_x));
+  } else if (dtype == JTMOE_BF16) {
+    dim3 block(64, 4);
+    const int grid = (int)((T + block.y - 1) / block.y);
+    dispatch_rows_kernel<uint16_t><<<grid, block, 0, s>>>(static_cast<const uint16_t*>(x), inverse, (int)T, (int)K,
+                                                          (int)A, (int)H, static_cast<uint16_t*>(packed_x));
+  } else {
+    dim3 block(64, 4);
+    const int grid = (int)((T + block.y - 1) / block.y);
+    dispatch_rows_kernel<uint32_t><<<grid, block, 0, s>>>(static_cast<const uint32_t*>(x), inverse, (int)T, (int)K,
+                                                          (int)A, (int)H, static_cast<uint32_t*>(packed_x));
+  }
+}
+
 }  // namespace jtmoe
 
 using namespace jtmoe;
@@ -210,30 +240,7 @@ extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t 
     dispatch_rank_kernel<<<nchunks, kDispThreads, (size_t)E * (1 + kDispWaves) * sizeof(int), s>>>(
         expert_ids, (int)A, (int)E, nchunks, partial, source_order, inverse);
     stage_mark(kStageDispatchMeta, s);
-    if (x != nullptr) {
-      const size_t row_bytes = (size_t)H * dtype_bytes(dtype);
-      const bool vec16 = row_bytes % 16 == 0 && aligned16(x) && aligned16(packed_x);
-      if (vec16) {
-        const int row_vecs = (int)(row_bytes / 16);
-        // one wave per row for short rows, up to 256 lanes for long ones
-        int bx = 64;
-        while (bx < 256 && bx * 4 < row_vecs) bx *= 2;
-        dim3 block(bx, 256 / bx);
-        const int grid = (int)((T + block.y - 1) / block.y);
-        dispatch_rows_kernel<uint4><<<grid, block, 0, s>>>(static_cast<const uint4*>(x), inverse, (int)T, (int)K,
-                                                           (int)A, row_vecs, static_cast<uint4*>(packed_x));
-      } else if (dtype == JTMOE_BF16) {
-        dim3 block(64, 4);
-        const int grid = (int)((T + block.y - 1) / block.y);
-        dispatch_rows_kernel<uint16_t><<<grid, block, 0, s>>>(static_cast<const uint16_t*>(x), inverse, (int)T, (int)K,
-                                                              (int)A, (int)H, static_cast<uint16_t*>(packed_x));
-      } else {
-        dim3 block(64, 4);
-        const int grid = (int)((T + block.y - 1) / block.y);
-        dispatch_rows_kernel<uint32_t><<<grid, block, 0, s>>>(static_cast<const uint32_t*>(x), inverse, (int)T, (int)K,
-                                                              (int)A, (int)H, static_cast<uint32_t*>(packed_x));
-      }
-    }
+    if (x != nullptr) launch_dispatch_rows(x, inverse, T, K, H, dtype, packed_x, s);
   }
   if (A == 0) stage_mark(kStageDispatchMeta, s);
   stage_mark(kStageDispatchRows, s);

@@ -449,7 +449,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
 
 // Configurations the library launches.
 using DgradCfg = NtGemmCfg<256, 256, 2, 4, 16 + 64>;   // data gradients: 256 x 256 tiles
-using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16 + 128>;  // gate and up weight gradients share the x tile
-using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16 + 128>;     // down weight gradient
+// narrow LDS blocks: the fastest layout when the operands are streamed (1.52 vs 1.60 ms for the
+// gate/up product of the C3 shape); the wide blocks pay off only when rows are gathered
+using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16>;  // gate and up weight gradients share the x tile
+using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16>;     // down weight gradient
 
 }  // namespace jtmoe

@@ -373,6 +373,14 @@ static void time_backward() {
     CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
     time_launches("wgrad gate/up (gathered x^T @ dG, dU)", 4.0 * rows * H * I, 10,
                   [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, true, false, false); });
+    {  // the same product on a permuted copy of x: what the library runs
+      uint16_t* Xp = random_bf16((size_t)rows * H, 36, 1.0f);
+      Problem q = p;
+      q.A = Xp;
+      time_launches("wgrad gate/up (packed x^T @ dG, dU)", 4.0 * rows * H * I, 10,
+                    [&] { launch_tn<WgradDualCfg>(q, D0, D1, C0, C1, false, false, false); });
+      hipFree(Xp);
+    }
     hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1);
     release(p);
   }
@@ -393,6 +401,12 @@ static void time_backward() {
     q.A = P;
     time_launches("wgrad down (act^T @ gathered dy)", 2.0 * rows * H * I, 10,
                   [&] { launch_tn<WgradCfg>(q, D, nullptr, C0, nullptr, false, true, false); });
+    {
+      uint16_t* dYp = random_bf16((size_t)rows * H, 37, 1.0f);
+      time_launches("wgrad down (act^T @ packed dy)", 2.0 * rows * H * I, 10,
+                    [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+      hipFree(dYp);
+    }
     hipFree(P); hipFree(D); hipFree(C0);
     release(p);
   }
