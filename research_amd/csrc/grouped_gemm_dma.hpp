@@ -11,8 +11,11 @@
 // are stored without padding and bank conflicts are avoided by permuting the
 // 16-byte chunks inside each row (an XOR swizzle applied to the *source* chunk):
 //   A tile [BM][BK]:        chunk c of row r sits in slot c ^ ((r / (16/CPR)) % CPR)
-//   B tile [BK][128] x NSUB: stored as 128-byte blocks of 4 k rows x 16 columns, so that
-//                            a 16-lane transposing read touches 128 contiguous bytes
+//   B tile [BK][128] x NSUB: stored as blocks of 4 k rows x 16 columns (128 bytes, one
+//                            16-lane transposing read touches one block) or, in the large
+//                            configurations, 4 k rows x 64 columns (512 bytes: eight lanes
+//                            fetch a whole 128-byte line; rows 2 and 3 keep their 64-byte
+//                            halves swapped so a transposing read meets no bank twice)
 // A fragments are read with ds_read_b128, B fragments with the transposing
 // ds_read_b64_tr_b16 (lane i of a 16-lane group addresses row i/4, columns
 // 4*(i%4)..; lane j receives the four k values of its column j).
@@ -167,10 +170,15 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     }
   }
   // B sub-tile [BK][128]: stored as 128-byte blocks of 4 k rows x 16 columns, block (k/4, n/16) at
-  // index (k/4)*8 + n/16; slot s (16 bytes) -> block s/8, row (s/2)%4 of the block, half s%2
-  const int b_blk_id = tid >> 3;
-  const int b_k = (b_blk_id >> 3) * 4 + ((tid >> 1) & 3);
-  const int b_c = (b_blk_id & 7) * 2 + (tid & 1);
+  // index (k/4)*8 + n/16; slot s (16 bytes) -> block s/8, row (s/2)%4 of the block, half s%2.
+  // OPT & 128: 512-byte blocks of 4 k rows x 64 columns instead (block (k/4, n/64) at index
+  // (k/4)*2 + n/64, slot s -> block s/32, row (s/8)%4, chunk s%8), so that eight lanes fetch one
+  // whole 128-byte line of the matrix; rows 2 and 3 of a block hold their two 64-byte halves
+  // swapped, which keeps the four 32-byte pieces of a transposing read in different banks.
+  constexpr bool kWide = (Cfg::OPT & 128) != 0;
+  const int b_blk_id = kWide ? tid >> 5 : tid >> 3;
+  const int b_k = kWide ? (b_blk_id >> 1) * 4 + ((tid >> 3) & 3) : (b_blk_id >> 3) * 4 + ((tid >> 1) & 3);
+  const int b_c = kWide ? (b_blk_id & 1) * 8 + ((tid & 7) ^ (((tid >> 4) & 1) << 2)) : (b_blk_id & 7) * 2 + (tid & 1);
   int b_voff[Cfg::NSUB];
 #pragma unroll
   for (int u = 0; u < Cfg::NSUB; ++u) b_voff[u] = (b_k * N + n0 + (kDual ? 0 : u * 128) + b_c * 8) * 2;
@@ -205,7 +213,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   const int a_rowoff = a_row * (BK * 2);
   // transposing read: the 16 lanes of a group read one whole 128-byte block, lane i its bytes
   // [8 i, 8 i + 8) = row i/4, columns 4*(i%4)..; groups: column half (lane/16)%2, k half lane/32
-  const int b_laneoff = (lane & 15) * 8 + ((lane >> 4) & 1) * 128 + (lane >> 5) * (2 * 8 * 128);
+  const int b_laneoff = kWide ? ((lane & 15) >> 2) * 128 + (lane & 3) * 8 + ((lane >> 4) & 1) * 32 + (lane >> 5) * 2048
+                              : (lane & 15) * 8 + ((lane >> 4) & 1) * 128 + (lane >> 5) * (2 * 8 * 128);
+  const int half_swap = kWide ? ((lane >> 3) & 1) * 64 : 0;  // the swapped halves, seen from the reading lane
   int b_blk[TN];  // byte offset of column block jj: sub-tile base + its first 16-column block
 #pragma unroll
   for (int jj = 0; jj < TN; ++jj) {
@@ -214,8 +224,12 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
       col = (jj < TN / 2 ? 0 : BN) + wn * (WN / 2) + (jj % (TN / 2)) * 32;
     else
       col = wn * WN + jj * 32;
-    const int u = col >> 7, nblk = (col & 127) >> 4;
-    b_blk[jj] = Cfg::A_BYTES + u * Cfg::BSUB_BYTES + nblk * 128;
+    const int u = col >> 7;
+    if (kWide)
+      b_blk[jj] = Cfg::A_BYTES + u * Cfg::BSUB_BYTES + ((col & 127) >> 6) * 512 + (col & 63) * 2 +
+                  ((col & 32) ? -half_swap : half_swap);
+    else
+      b_blk[jj] = Cfg::A_BYTES + u * Cfg::BSUB_BYTES + ((col & 127) >> 4) * 128;
   }
 
   auto load_frags = [&](const unsigned char* st, int kk, bf16x8_t* af, bf16x8_t* bf) {
@@ -327,14 +341,15 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
 }
 
 // The two configurations the library launches: 256 x 256 output tiles (gate and up share the A
-// tile: 128 + 128 columns), 64-deep k steps, two LDS stages, 8 waves.
-using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16>;
-using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64>;
+// tile: 128 + 128 columns), 64-deep k steps, two LDS stages, 8 waves, B tiles in 4 x 64 blocks
+// (whole 128-byte lines per eight lanes: 3 % and 7 % faster than 4 x 16 blocks at 131072 rows).
+using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
+using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128>;
 // Few rows per group (decode-sized batches): the layer streams every expert matrix once and
 // is bound by HBM, so the tiles are only 64 rows tall to keep the padded-row MFMA work below
 // the time the weights take to arrive.  Several workgroups share a CU, so that one computes
 // while another waits for its tiles.
-using GateUpSmallCfg = DmaGemmCfg<64, 128, 64, 2, 4, true, 2, 16>;
+using GateUpSmallCfg = DmaGemmCfg<64, 128, 64, 2, 4, true, 2, 16 + 128>;
 using DownSmallCfg = DmaGemmCfg<64, 256, 32, 1, 4, false, 2, 16>;  // four workgroups of four waves per CU
 
 }  // namespace jtmoe

@@ -476,6 +476,15 @@ int main(int argc, char** argv) {
     ok &= check_tn<WgradDualCfg>("wgrad dual dense", p, 0, true);
     release(p);
   }
+  {
+    // the 4 x 16 block layout of the B tile, which the large configurations no longer use
+    using GateUpNarrowCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16>;
+    using DownNarrowCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64>;
+    Problem p = make(7, 3001, 576, 392, 21, true, 0, 1.0f);
+    ok &= check<GateUpNarrowCfg>("gate/up ragged, 4 x 16 blocks", p);
+    ok &= check<DownNarrowCfg>("down ragged, 4 x 16 blocks", p);
+    release(p);
+  }
   if (ok && argc > 1 && !strcmp(argv[1], "time_backward")) time_backward();
   if (ok && argc > 1 && !strcmp(argv[1], "time_decode")) time_decode();
   if (ok && argc > 1 && !strcmp(argv[1], "time")) {
