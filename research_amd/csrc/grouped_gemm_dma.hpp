@@ -342,7 +342,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
 
 // The two configurations the library launches: 256 x 256 output tiles (gate and up share the A
 // tile: 128 + 128 columns), 64-deep k steps, two LDS stages, 8 waves, B tiles in 4 x 64 blocks
-// (whole 128-byte lines per eight lanes: 3 % and 7 % faster than 4 x 16 blocks at 131072 rows).
+// (whole 128-byte lines per eight lanes; about 1 % faster than 4 x 16 blocks at 131072 rows).
 using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
 using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128>;
 // Few rows per group (decode-sized batches): the layer streams every expert matrix once and

@@ -164,7 +164,9 @@ template <typename Cfg>
 static void timeit(const char* name, Problem& p, int iters) {
   hipEvent_t a, b;
   CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
-  for (int i = 0; i < 10; ++i) launch<Cfg>(p, false);
+  // a long warm-up: the first tens of milliseconds after a pause on the host side (here, filling
+  // the operands) run several per cent slower, whichever kernel is timed
+  for (int i = 0; i < 60; ++i) launch<Cfg>(p, false);
   CK(hipDeviceSynchronize());
   CK(hipEventRecord(a));
   for (int i = 0; i < iters; ++i) launch<Cfg>(p, false);
@@ -330,7 +332,7 @@ template <typename F>
 static void time_launches(const char* name, double flops, int iters, F launch_once) {
   hipEvent_t a, b;
   CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
-  for (int i = 0; i < 5; ++i) launch_once();
+  for (int i = 0; i < 40; ++i) launch_once();  // long warm-up, as in timeit
   CK(hipDeviceSynchronize());
   CK(hipEventRecord(a));
   for (int i = 0; i < iters; ++i) launch_once();
