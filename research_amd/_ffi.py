@@ -117,7 +117,8 @@ STAGE_NAMES = (
 JTMOE_BF16 = 0
 JTMOE_F32 = 1
 
-_LOADED_LIBS: dict[str, ctypes.CDLL] = {}
+_LOADED_LIBS: dict[str, ctypes.CDLL] = {}  # by path of the shared object
+_LIBS_BY_ROOT: dict[str, ctypes.CDLL] = {}  # by cache root, once its manifest and checksum have been validated
 
 
 def shared_object_path(cache_root: str | Path | None = None) -> Path:
@@ -147,10 +148,20 @@ def shared_object_path(cache_root: str | Path | None = None) -> Path:
 
 
 def load_library(cache_root: str | Path | None = None) -> ctypes.CDLL:
-    """Open libjtmoe.so (once per path) and attach the prototypes."""
+    """Open libjtmoe.so and attach the prototypes.
+
+    The manifest and the checksum are validated when a cache root is first used in the process, as the
+    reference does at registration (_ffi.py:19-45); later calls return the library already opened
+    (hashing the file again on every operator call would cost more than a small layer call itself).
+    """
+    root_key = "" if cache_root is None else Path(cache_root).as_posix()
+    cached = _LIBS_BY_ROOT.get(root_key)
+    if cached is not None:
+        return cached
     path = shared_object_path(cache_root)
     key = path.as_posix()
     if key in _LOADED_LIBS:
+        _LIBS_BY_ROOT[root_key] = _LOADED_LIBS[key]
         return _LOADED_LIBS[key]
     try:
         library = ctypes.CDLL(key)
@@ -164,6 +175,7 @@ def load_library(cache_root: str | Path | None = None) -> ctypes.CDLL:
         fn.restype = restype
         fn.argtypes = argtypes
     _LOADED_LIBS[key] = library
+    _LIBS_BY_ROOT[root_key] = library
     return library
 
 
@@ -174,3 +186,4 @@ def last_error(library: ctypes.CDLL) -> str:
 
 def reset_registrations_for_tests() -> None:
     _LOADED_LIBS.clear()
+    _LIBS_BY_ROOT.clear()

@@ -136,6 +136,19 @@ def test_loader_refuses_missing_or_stale_artifacts(tmp_path):
         _ffi.shared_object_path(tmp_path)
 
 
+def test_library_is_validated_once_per_process_not_per_call(monkeypatch):
+    _ffi.reset_registrations_for_tests()
+    calls = []
+    real = _ffi._sha256
+    monkeypatch.setattr(_ffi, "_sha256", lambda path: (calls.append(path), real(path))[1])
+    first = _ffi.load_library()
+    assert len(calls) == 1
+    for _ in range(3):
+        assert _ffi.load_library() is first
+    assert len(calls) == 1  # operator calls after the first do not hash the file again
+    assert _ffi.load_library(build.cache_dir()) is first and len(calls) == 2  # another spelling of the root: checked, same handle
+
+
 def test_manifest_records_the_build():
     manifest = build.load_cache_manifest()
     art = manifest["artifacts"]["moe"]["ffi"]
