@@ -141,6 +141,92 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_rank_kernel(const int32
   }
 }
 
+// Small batches: the three passes in one workgroup of 1024 threads (histogram in LDS, scan over the
+// experts with wave shuffles, then the same ballot ranking with 16 waves per round of 1024
+// assignments).  At a few hundred assignments the three launches above are idle most of their
+// time; this is one launch with the same results.
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallWaves = kSmallThreads / kWave;
+constexpr int kSmallMaxAssignments = 8192;
+constexpr int kSmallMaxExperts = JTMOE_MAX_EXPERTS;  // one thread per expert in the scan
+__global__ __launch_bounds__(kSmallThreads) void dispatch_small_kernel(const int32_t* __restrict__ ids, int A, int E,
+                                                                      int32_t* __restrict__ group_sizes,
+                                                                      int32_t* __restrict__ offsets,
+                                                                      int32_t* __restrict__ source_order,
+                                                                      int32_t* __restrict__ inverse) {
+  extern __shared__ int smem[];
+  int* cursor = smem;        // [E] histogram, then the next free packed row of expert e
+  int* wavehist = smem + E;  // [kSmallWaves][E]
+  __shared__ int wave_sums[kSmallWaves];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  for (int e = tid; e < E; e += kSmallThreads) cursor[e] = 0;
+  for (int i = tid; i < kSmallWaves * E; i += kSmallThreads) wavehist[i] = 0;
+  __syncthreads();
+  for (int a = tid; a < A; a += kSmallThreads) {
+    const int id = ids[a];
+    if (id >= 0 && id < E) atomicAdd(&cursor[id], 1);
+  }
+  __syncthreads();
+  // exclusive scan over the experts: thread e owns expert e (E <= 1024 threads)
+  const int count = tid < E ? cursor[tid] : 0;
+  int incl = count;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int v = __shfl_up(incl, d);
+    if (lane >= d) incl += v;
+  }
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  int before = 0;
+  for (int w = 0; w < wave; ++w) before += wave_sums[w];
+  const int start = incl + before - count;
+  if (tid < E) {
+    offsets[tid] = start;
+    group_sizes[tid] = count;
+    cursor[tid] = start;
+  }
+  __syncthreads();
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  for (int base = 0; base < A; base += kSmallThreads) {
+    const int a = base + tid;
+    int id = -1;
+    if (a < A) {
+      id = ids[a];
+      if (id < 0 || id >= E) id = -1;
+    }
+    const bool valid = id >= 0;
+    unsigned long long peers = __ballot(valid);  // lanes of this wave holding the same expert id
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (id >> b) & 1;
+      const unsigned long long m = __ballot(valid && bit);
+      peers &= bit ? m : ~m;
+    }
+    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+    if (valid && rank == 0) wavehist[wave * E + id] = __popcll(peers);
+    __syncthreads();
+    if (valid) {
+      int pos = cursor[id] + rank;
+      for (int w = 0; w < wave; ++w) pos += wavehist[w * E + id];
+      inverse[a] = pos;
+      source_order[pos] = a;
+    } else if (a < A) {
+      inverse[a] = -1;
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += kSmallThreads) {
+      int add = 0;
+#pragma unroll
+      for (int w = 0; w < kSmallWaves; ++w) {
+        add += wavehist[w * E + e];
+        wavehist[w * E + e] = 0;
+      }
+      cursor[e] += add;
+    }
+    __syncthreads();
+  }
+}
+
 // pass 4: token-major row scatter; each token row is read once and written to
 // its K packed positions.  V is the vector type moved per lane.
 template <typename V>
@@ -231,6 +317,14 @@ extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t 
     return fail(JTMOE_EWORKSPACE, "dispatch: workspace %zu < %zu bytes", workspace_bytes,
                 jtmoe_dispatch_workspace_bytes(A, E));
   hipStream_t s = as_stream(stream);
+  if (A > 0 && A <= kSmallMaxAssignments && E <= kSmallMaxExperts) {
+    dispatch_small_kernel<<<1, kSmallThreads, (size_t)E * (1 + kSmallWaves) * sizeof(int), s>>>(
+        expert_ids, (int)A, (int)E, group_sizes, offsets, source_order, inverse);
+    stage_mark(kStageDispatchMeta, s);
+    if (x != nullptr) launch_dispatch_rows(x, inverse, T, K, H, dtype, packed_x, s);
+    stage_mark(kStageDispatchRows, s);
+    return check_launch("dispatch");
+  }
   const int nchunks = dispatch_chunks(A > 0 ? A : 1);
   int* partial = static_cast<int*>(workspace);
   dispatch_hist_kernel<<<nchunks, kDispThreads, (size_t)E * sizeof(int), s>>>(expert_ids, (int)A, (int)E, nchunks,

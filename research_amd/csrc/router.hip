@@ -65,6 +65,8 @@ __host__ __device__ inline RouterScratch router_scratch(void* ws, int E) {
   return s;
 }
 
+inline size_t router_scratch_bytes(int64_t E) { return align_up((size_t)E * 12, 256); }
+
 __global__ void router_zero_kernel(void* ws, int E) {
   RouterScratch s = router_scratch(ws, E);
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
@@ -112,13 +114,58 @@ __device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, in
   return s;
 }
 
+// K rounds of "largest remaining score + bias, lower index on ties" for one token, by its four
+// lanes: lane q owns experts [e_begin, e_begin + EQ) and keeps them in registers.
+template <int EQ>
+__device__ __forceinline__ void select_from_registers(const RouterSmem& sm, const float* row, int e_begin, bool row_ok,
+                                                      int t, int q, int K) {
+#pragma clang fp contract(off)
+  float v[EQ];
+#pragma unroll
+  for (int j = 0; j < EQ; ++j) v[j] = row_ok ? row[e_begin + j] + sm.bias[e_begin + j] : 0.0f;
+  unsigned long long taken = 0ull;
+  for (int r = 0; r < K; ++r) {
+    float best_v = 0.0f;
+    int best_e = -1;
+    if (row_ok) {
+#pragma unroll
+      for (int j = 0; j < EQ; ++j) {
+        if (!((taken >> j) & 1ull) && (best_e < 0 || v[j] > best_v)) {
+          best_v = v[j];
+          best_e = e_begin + j;
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 1; m <= 2; m <<= 1) {
+      const float ov = __shfl_xor(best_v, m, 4);
+      const int oe = __shfl_xor(best_e, m, 4);
+      const bool take = oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e));
+      if (take) {
+        best_v = ov;
+        best_e = oe;
+      }
+    }
+    if (row_ok) {
+      const int j = best_e - e_begin;
+      if (j >= 0 && j < EQ) taken |= 1ull << j;
+      if (q == 0) {
+        sm.top_id[t * K + r] = best_e;
+        sm.top_score[t * K + r] = row[best_e];
+      }
+    }
+  }
+}
+
 // Everything after the logits tile is in LDS.  `T` is the output element type of
 // the weights.
 template <typename T, int kRouterTokens, int kRouterThreads>
 __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ bias_g, int t0, int tokens,
                                 int E, int K, float route_scale, int32_t* __restrict__ ids_out,
                                 T* __restrict__ weights_out, float* __restrict__ scores_out,
-                                float* __restrict__ logits_out, RouterScratch g) {
+                                float* __restrict__ logits_out, RouterScratch g,
+                                float* __restrict__ counts_final = nullptr,
+                                float* __restrict__ importance_final = nullptr) {
 #pragma clang fp contract(off)
   const int tid = threadIdx.x;
   const int stride = E + 1;
@@ -145,8 +192,19 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
   const int eq = (E + 3) >> 2;
   const int e_begin = q * eq;
   const bool row_ok = t < nrows;
-  unsigned long long taken = 0ull;
   const float* row = sm.tile + t * stride;
+  // For the usual expert counts the lane keeps its quarter (score + bias) in registers, so that a
+  // round is a run of compares instead of a chain of LDS reads; same scan order, same comparisons.
+  if (E == 64 || E == 128 || E == 32 || E == 256 || E == 16) {
+    switch (E) {
+      case 16: select_from_registers<4>(sm, row, e_begin, row_ok, t, q, K); break;
+      case 32: select_from_registers<8>(sm, row, e_begin, row_ok, t, q, K); break;
+      case 64: select_from_registers<16>(sm, row, e_begin, row_ok, t, q, K); break;
+      case 128: select_from_registers<32>(sm, row, e_begin, row_ok, t, q, K); break;
+      default: select_from_registers<64>(sm, row, e_begin, row_ok, t, q, K); break;
+    }
+  } else {
+  unsigned long long taken = 0ull;
   for (int r = 0; r < K; ++r) {
     float best_v = 0.0f;
     int best_e = -1;
@@ -181,6 +239,7 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
       }
     }
   }
+  }
   // renormalise (lane 0 of the token; it wrote top_* itself)
   if (row_ok && q == 0) {
     float denom = sm.top_score[t * K];
@@ -199,6 +258,14 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
     }
   }
   __syncthreads();
+  if (counts_final != nullptr) {
+    // the only workgroup of the call: its sums are the statistics (same conversion as router_finalize_kernel)
+    for (int e = tid; e < E; e += kRouterThreads) {
+      counts_final[e] = (float)sm.cnt[e];
+      importance_final[e] = (float)((double)sm.imp[e] * (1.0 / 4294967296.0));
+    }
+    return;
+  }
   for (int e = tid; e < E; e += kRouterThreads) {
     const int c = sm.cnt[e];
     if (c) {
@@ -426,11 +493,15 @@ __host__ __device__ inline size_t router_split_smem_bytes(int E, int K) {
   return w > ep ? w : ep;
 }
 
-template <int NB>
+// kPartial: the grid's y dimension also shares out the chunks (chunks_per_slice each); a workgroup
+// then only writes its unrounded partial sums, partial_out[slice][token][expert], and
+// router_finish_kernel adds the slices in order and does the rest.
+template <int NB, bool kPartial>
 __global__ __launch_bounds__(256) void router_mfma_split_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
     int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
-    float* __restrict__ scores, float* __restrict__ logits_out, void* ws) {
+    float* __restrict__ scores, float* __restrict__ logits_out, void* ws, float* __restrict__ partial_out,
+    int chunks_per_slice) {
   constexpr int kThreads = 256, kTokens = 16;
   constexpr int E = NB * 16;
   constexpr int WS = E + 32;
@@ -479,10 +550,13 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
 
   // transposing read: the 16-lane group kg reads rows wave*32 + kg*8 + 4*h + i/4, columns 4*(i%4)..
   const int w_lane = (wave * 32 + (lane >> 4) * 8 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
-  const int nchunks = H / kSplitKC;
+  // this workgroup's chunks: all of them, or one slice of them
+  const int chunk0 = kPartial ? (int)blockIdx.y * chunks_per_slice : 0;
+  const int nchunks = kPartial ? min(chunks_per_slice, H / kSplitKC - chunk0) : H / kSplitKC;
+  const int kbase = chunk0 * kSplitKC;
 #pragma unroll
   for (int d = 0; d < D; ++d)
-    if (d < nchunks) JT_LOAD(d, d * kSplitKC);
+    if (d < nchunks) JT_LOAD(d, kbase + d * kSplitKC);
   JT_STORE_W(0, 0);
   __syncthreads();
   for (int kc0 = 0; kc0 < nchunks; kc0 += UNROLL) {
@@ -503,7 +577,7 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
           acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
         }
         if (kc + 1 < nchunks) JT_STORE_W(next_slot, stage ^ 1);
-        if (kc + D < nchunks) JT_LOAD(slot, (kc + D) * kSplitKC);
+        if (kc + D < nchunks) JT_LOAD(slot, kbase + (kc + D) * kSplitKC);
         __syncthreads();
       }
     }
@@ -527,11 +601,45 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
     float v = red[t * stride + e];
 #pragma unroll
     for (int wv = 1; wv < 4; ++wv) v += red[(wv * kTokens + t) * stride + e];
-    sm.tile[t * stride + e] = round_to_bf16(v);
+    if (kPartial) {
+      if (t < nrows) partial_out[((size_t)blockIdx.y * tokens + t0 + t) * E + e] = v;
+    } else {
+      sm.tile[t * stride + e] = round_to_bf16(v);
+    }
   }
+  if (kPartial) return;
   __syncthreads();
   router_epilogue<bf16_raw, kTokens, kThreads>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores,
                                                logits_out, router_scratch(ws, E));
+}
+
+// Second half of the small-batch router: one workgroup adds the slices of partial sums in slice
+// order, rounds to bf16 (the projection's output dtype) and runs the epilogue for every token of
+// the call, so the statistics need neither the zeroing nor the finalising launch.
+constexpr int kPartialMaxSlices = 16;
+template <int kTok>
+__global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
+    const float* __restrict__ partial, int slices, const float* __restrict__ bias, int tokens, int E, int K,
+    float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights, float* __restrict__ scores,
+    float* __restrict__ logits_out, float* __restrict__ counts, float* __restrict__ importance) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  RouterSmem sm = router_smem(smem_raw, E, K, kTok);
+  const int stride = E + 1;
+  const size_t plane = (size_t)tokens * E;
+  for (int idx = threadIdx.x; idx < tokens * E; idx += 4 * kTok) {
+    const int t = idx / E, e = idx - t * E;
+    float part[kPartialMaxSlices];  // all slices requested before the first is needed
+#pragma unroll
+    for (int sl = 0; sl < kPartialMaxSlices; ++sl) part[sl] = sl < slices ? partial[sl * plane + idx] : 0.0f;
+    float v = part[0];
+#pragma unroll
+    for (int sl = 1; sl < kPartialMaxSlices; ++sl)
+      if (sl < slices) v += part[sl];
+    sm.tile[t * stride + e] = round_to_bf16(v);
+  }
+  __syncthreads();
+  router_epilogue<bf16_raw, kTok, 4 * kTok>(sm, bias, 0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
+                                            RouterScratch{}, counts, importance);
 }
 
 template <typename KernelT>
@@ -560,16 +668,57 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
       const size_t smem = router_split_smem_bytes((int)E, (int)K);
       if (smem > 160 * 1024)
         return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
+      // Two launches when one workgroup can hold the epilogue of the whole call: partial sums over
+      // k slices from many workgroups, then the finishing workgroup.
+      const int finish_tok = router_smem_bytes((int)E, (int)K, 256) <= 160 * 1024 ? 256 : 64;
+      if (tokens > 0 && tokens <= finish_tok && router_smem_bytes((int)E, (int)K, finish_tok) <= 160 * 1024) {
+        const int chunks = (int)(H / kSplitKC);
+        const int per_slice = (chunks + kPartialMaxSlices - 1) / kPartialMaxSlices;
+        const int slices = (chunks + per_slice - 1) / per_slice;
+        float* partial = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + router_scratch_bytes(E));
+#define JT_PARTIAL_CASE(NB)                                                                                   \
+  case NB * 16: {                                                                                            \
+    auto kernel = router_mfma_split_kernel<NB, true>;                                                        \
+    int rc = set_max_smem(kernel, smem);                                                                     \
+    if (rc) return rc;                                                                                       \
+    kernel<<<dim3(blocks, slices), 256, smem, stream>>>(                                                     \
+        static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws, partial, per_slice); \
+  } break;
+        switch ((int)E) {
+          JT_PARTIAL_CASE(1)
+          JT_PARTIAL_CASE(2)
+          JT_PARTIAL_CASE(4)
+          JT_PARTIAL_CASE(8)
+          JT_PARTIAL_CASE(16)
+        }
+#undef JT_PARTIAL_CASE
+        const size_t fsmem = router_smem_bytes((int)E, (int)K, finish_tok);
+        if (finish_tok == 256) {
+          auto kernel = router_finish_kernel<256>;
+          int rc = set_max_smem(kernel, fsmem);
+          if (rc) return rc;
+          kernel<<<1, 1024, fsmem, stream>>>(partial, slices, bias, (int)tokens, (int)E, (int)K, (float)route_scale, ids,
+                                             static_cast<bf16_raw*>(weights), scores, logits_out, counts, importance);
+        } else {
+          auto kernel = router_finish_kernel<64>;
+          int rc = set_max_smem(kernel, fsmem);
+          if (rc) return rc;
+          kernel<<<1, 256, fsmem, stream>>>(partial, slices, bias, (int)tokens, (int)E, (int)K, (float)route_scale, ids,
+                                            static_cast<bf16_raw*>(weights), scores, logits_out, counts, importance);
+        }
+        return check_launch("router");
+      }
       router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
       if (tokens > 0) {
 #define JT_SPLIT_CASE(NB)                                                                                     \
   case NB * 16: {                                                                                            \
-    auto kernel = router_mfma_split_kernel<NB>;                                                              \
+    auto kernel = router_mfma_split_kernel<NB, false>;                                                       \
     int rc = set_max_smem(kernel, smem);                                                                     \
     if (rc) return rc;                                                                                       \
     kernel<<<blocks, 256, smem, stream>>>(                                                                   \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws);                   \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws, nullptr, 0);       \
   } break;
         switch ((int)E) {
           JT_SPLIT_CASE(1)
@@ -652,7 +801,8 @@ using namespace jtmoe;
 
 extern "C" size_t jtmoe_router_workspace_bytes(int64_t E) {
   if (E <= 0) return 0;
-  return align_up((size_t)E * 12, 256);
+  // the statistics accumulators, then the partial sums of the small-batch path
+  return router_scratch_bytes(E) + align_up((size_t)kPartialMaxSlices * kSplitMaxTokens * E * sizeof(float), 256);
 }
 
 extern "C" int jtmoe_router(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H,

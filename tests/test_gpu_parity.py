@@ -123,7 +123,11 @@ def check_router_end_to_end(gpu, x, w, bias, top_k, scale, dtype):
 @pytest.mark.parametrize(
     "tokens,hidden,experts,top_k,dtype",
     [(64, 32, 8, 2, "f32"), (257, 512, 8, 2, "f32"), (300, 1024, 16, 2, "bf16"), (1024, 2048, 64, 8, "bf16"),
-     (513, 2048, 128, 8, "bf16"), (100, 72, 24, 3, "bf16")],
+     (513, 2048, 128, 8, "bf16"), (100, 72, 24, 3, "bf16"),
+     # small batches: k-sliced partial sums + one finishing workgroup (256- and 64-token forms), the
+     # uneven last slice, and the shape that falls back to the 16-token workgroups
+     (64, 2048, 64, 8, "bf16"), (1, 256, 16, 1, "bf16"), (256, 1024, 128, 8, "bf16"), (64, 512, 256, 4, "bf16"),
+     (17, 2176, 32, 2, "bf16"), (255, 512, 256, 4, "bf16")],
 )
 def test_router_end_to_end(gpu, tokens, hidden, experts, top_k, dtype):
     rng = np.random.default_rng(hidden + experts)
@@ -151,7 +155,9 @@ def check_dispatch(gpu, ids: np.ndarray, experts: int, x: np.ndarray | None, dty
 @pytest.mark.parametrize(
     "tokens,top_k,experts,hidden,dtype",
     [(1, 1, 1, 8, "f32"), (6, 2, 4, 3, "f32"), (511, 2, 8, 64, "bf16"), (512, 2, 8, 64, "bf16"), (513, 2, 8, 64, "bf16"),
-     (1000, 8, 64, 256, "bf16"), (4096, 8, 128, 40, "bf16"), (333, 3, 256, 7, "bf16"), (2048, 2, 16, 1024, "f32")],
+     (1000, 8, 64, 256, "bf16"), (4096, 8, 128, 40, "bf16"), (333, 3, 256, 7, "bf16"), (2048, 2, 16, 1024, "f32"),
+     # either side of the single-workgroup limit (8192 assignments)
+     (1024, 8, 32, 8, "bf16"), (8193, 1, 32, 8, "bf16"), (700, 4, 256, 8, "bf16")],
 )
 def test_dispatch_is_bit_exact(gpu, tokens, top_k, experts, hidden, dtype):
     rng = np.random.default_rng(tokens + experts)
