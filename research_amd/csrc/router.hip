@@ -114,6 +114,19 @@ __device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, in
   return s;
 }
 
+// Exchange inside an aligned group of four lanes (lane ^ 1 and lane ^ 2) as a DPP register move
+// instead of a trip through the LDS crossbar.
+template <int kXor>
+__device__ __forceinline__ int quad_xor_i32(int v) {
+  static_assert(kXor == 1 || kXor == 2, "quad exchange");
+  return kXor == 1 ? __builtin_amdgcn_mov_dpp(v, 0xB1, 0xf, 0xf, true)   // quad_perm [1,0,3,2]
+                   : __builtin_amdgcn_mov_dpp(v, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+}
+template <int kXor>
+__device__ __forceinline__ float quad_xor_f32(float v) {
+  return __builtin_bit_cast(float, quad_xor_i32<kXor>(__builtin_bit_cast(int, v)));
+}
+
 // K rounds of "largest remaining score + bias, lower index on ties" for one token, by its four
 // lanes: lane q owns experts [e_begin, e_begin + EQ) and keeps them in registers.
 template <int EQ>
@@ -136,12 +149,18 @@ __device__ __forceinline__ void select_from_registers(const RouterSmem& sm, cons
         }
       }
     }
-#pragma unroll
-    for (int m = 1; m <= 2; m <<= 1) {
-      const float ov = __shfl_xor(best_v, m, 4);
-      const int oe = __shfl_xor(best_e, m, 4);
-      const bool take = oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e));
-      if (take) {
+    {
+      const float ov = quad_xor_f32<1>(best_v);
+      const int oe = quad_xor_i32<1>(best_e);
+      if (oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e))) {
+        best_v = ov;
+        best_e = oe;
+      }
+    }
+    {
+      const float ov = quad_xor_f32<2>(best_v);
+      const int oe = quad_xor_i32<2>(best_e);
+      if (oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e))) {
         best_v = ov;
         best_e = oe;
       }
@@ -626,6 +645,7 @@ __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
   RouterSmem sm = router_smem(smem_raw, E, K, kTok);
   const int stride = E + 1;
   const size_t plane = (size_t)tokens * E;
+#pragma unroll 4
   for (int idx = threadIdx.x; idx < tokens * E; idx += 4 * kTok) {
     const int t = idx / E, e = idx - t * E;
     float part[kPartialMaxSlices];  // all slices requested before the first is needed
