@@ -176,6 +176,47 @@ __device__ __forceinline__ void select_from_registers(const RouterSmem& sm, cons
   }
 }
 
+// The same selection for any expert count: the lane re-reads its quarter from LDS in every round.
+__device__ __forceinline__ void select_from_lds(const RouterSmem& sm, const float* row, int e_begin, int eq, int E,
+                                                bool row_ok, int t, int q, int K) {
+#pragma clang fp contract(off)
+  unsigned long long taken = 0ull;
+  for (int r = 0; r < K; ++r) {
+    float best_v = 0.0f;
+    int best_e = -1;
+    if (row_ok) {
+      for (int j = 0; j < eq; ++j) {
+        const int e = e_begin + j;
+        if (e < E && !((taken >> j) & 1ull)) {
+          const float v = row[e] + sm.bias[e];
+          if (best_e < 0 || v > best_v) {
+            best_v = v;
+            best_e = e;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 1; m <= 2; m <<= 1) {
+      const float ov = __shfl_xor(best_v, m, 4);
+      const int oe = __shfl_xor(best_e, m, 4);
+      const bool take = oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e));
+      if (take) {
+        best_v = ov;
+        best_e = oe;
+      }
+    }
+    if (row_ok) {
+      const int j = best_e - e_begin;
+      if (j >= 0 && j < eq) taken |= 1ull << j;
+      if (q == 0) {
+        sm.top_id[t * K + r] = best_e;
+        sm.top_score[t * K + r] = row[best_e];
+      }
+    }
+  }
+}
+
 // Everything after the logits tile is in LDS.  `T` is the output element type of
 // the weights.
 template <typename T, int kRouterTokens, int kRouterThreads>
@@ -223,41 +264,7 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
       default: select_from_registers<64>(sm, row, e_begin, row_ok, t, q, K); break;
     }
   } else {
-  unsigned long long taken = 0ull;
-  for (int r = 0; r < K; ++r) {
-    float best_v = 0.0f;
-    int best_e = -1;
-    if (row_ok) {
-      for (int j = 0; j < eq; ++j) {
-        const int e = e_begin + j;
-        if (e < E && !((taken >> j) & 1ull)) {
-          const float v = row[e] + sm.bias[e];
-          if (best_e < 0 || v > best_v) {
-            best_v = v;
-            best_e = e;
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int m = 1; m <= 2; m <<= 1) {
-      const float ov = __shfl_xor(best_v, m, 4);
-      const int oe = __shfl_xor(best_e, m, 4);
-      const bool take = oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e));
-      if (take) {
-        best_v = ov;
-        best_e = oe;
-      }
-    }
-    if (row_ok) {
-      const int j = best_e - e_begin;
-      if (j >= 0 && j < eq) taken |= 1ull << j;
-      if (q == 0) {
-        sm.top_id[t * K + r] = best_e;
-        sm.top_score[t * K + r] = row[best_e];
-      }
-    }
-  }
+    select_from_lds(sm, row, e_begin, eq, E, row_ok, t, q, K);
   }
   // renormalise (lane 0 of the token; it wrote top_* itself)
   if (row_ok && q == 0) {
