@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void swiglu_backward_bf16_vec_kernel(
   const size_t base = (size_t)j * row_vecs;
   float dot = 0.0f;
   for (int v = lane; v < row_vecs; v += 64) {
-    const uint4 zv = z_dg[base + v], gv = G[base + v], uv = U[base + v];
+    const uint4 zv = load_stream(&z_dg[base + v]), gv = load_stream(&G[base + v]), uv = load_stream(&U[base + v]);
     const uint32_t zw[4] = {zv.x, zv.y, zv.z, zv.w}, gw[4] = {gv.x, gv.y, gv.z, gv.w},
                    uw[4] = {uv.x, uv.y, uv.z, uv.w};
     uint32_t dgw[4], duw[4], hww[4];
@@ -108,9 +108,9 @@ __global__ __launch_bounds__(256) void swiglu_backward_bf16_vec_kernel(
       dot += lo.zh;
       dot += hi.zh;
     }
-    z_dg[base + v] = make_uint4(dgw[0], dgw[1], dgw[2], dgw[3]);
-    dU[base + v] = make_uint4(duw[0], duw[1], duw[2], duw[3]);
-    HW[base + v] = make_uint4(hww[0], hww[1], hww[2], hww[3]);
+    store_stream(&z_dg[base + v], make_uint4(dgw[0], dgw[1], dgw[2], dgw[3]));
+    store_stream(&dU[base + v], make_uint4(duw[0], duw[1], duw[2], duw[3]));
+    store_stream(&HW[base + v], make_uint4(hww[0], hww[1], hww[2], hww[3]));
   }
   dot = wave_sum(dot);
   if (row_weight_index && lane == 0) d_weights[a] = (uint16_t)f32_to_bf16_bits(dot);

@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void combine_bf16_vec_kernel(const uint4* __re
 #pragma unroll
       for (int j = 0; j < NV; ++j) {
         const int v = lane + j * 64;
-        rows[s][j] = (ok && v < row_vecs) ? packed_y[(size_t)pos[s] * row_vecs + v] : make_uint4(0, 0, 0, 0);
+        rows[s][j] = (ok && v < row_vecs) ? load_stream(&packed_y[(size_t)pos[s] * row_vecs + v]) : make_uint4(0, 0, 0, 0);
       }
     }
 #pragma unroll
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256) void combine_bf16_vec_kernel(const uint4* __re
 #pragma unroll
       for (int j = 0; j < NV; ++j) {
         const int v = lane + j * 64;
-        r[j] = v < row_vecs ? packed_y[(size_t)pos * row_vecs + v] : make_uint4(0, 0, 0, 0);
+        r[j] = v < row_vecs ? load_stream(&packed_y[(size_t)pos * row_vecs + v]) : make_uint4(0, 0, 0, 0);
       }
       add_row(r, w);
     }
@@ -127,12 +127,12 @@ __global__ __launch_bounds__(256) void combine_bf16_vec_kernel(const uint4* __re
     for (int i = 0; i < 8; ++i) acc[j][i] = round_bf16_hw(acc[j][i]);
     if (shared_y) {
       float f[8];
-      unpack8(shared_y[(size_t)t * row_vecs + v], f);
+      unpack8(load_stream(&shared_y[(size_t)t * row_vecs + v]), f);
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[j][i] = acc[j][i] + f[i];  // rounded by the packing
     }
     if (!kNorm) {
-      y[(size_t)t * row_vecs + v] = pack8_hw(acc[j]);
+      store_stream(&y[(size_t)t * row_vecs + v], pack8_hw(acc[j]));
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void combine_bf16_vec_kernel(const uint4* __re
       const int v = lane + j * 64;
       if (v >= row_vecs) continue;
       float r[8];
-      unpack8(residual[(size_t)t * row_vecs + v], r);
+      unpack8(load_stream(&residual[(size_t)t * row_vecs + v]), r);
       const float4 s0 = reinterpret_cast<const float4*>(post_scale)[v * 2];
       const float4 s1 = reinterpret_cast<const float4*>(post_scale)[v * 2 + 1];
       const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(256) void combine_bf16_vec_kernel(const uint4* __re
         const float n = round_bf16_hw(acc[j][i] * (inv * sc[i]));
         acc[j][i] = r[i] + n;  // rounded by the packing
       }
-      y[(size_t)t * row_vecs + v] = pack8_hw(acc[j]);
+      store_stream(&y[(size_t)t * row_vecs + v], pack8_hw(acc[j]));
     }
   }
 }

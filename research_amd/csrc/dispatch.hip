@@ -242,7 +242,7 @@ __global__ __launch_bounds__(256) void dispatch_rows_kernel(const V* __restrict_
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int v = v0 + j * blockDim.x;
-      if (v < row_vecs) r[j] = src[v];
+      if (v < row_vecs) r[j] = load_stream(&src[v]);
     }
     for (int s = 0; s < K; ++s) {
       const int pos = inverse[(size_t)t * K + s];
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(256) void dispatch_rows_kernel(const V* __restrict_
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int v = v0 + j * blockDim.x;
-        if (v < row_vecs) dst[v] = r[j];
+        if (v < row_vecs) store_stream(&dst[v], r[j]);
       }
     }
   }

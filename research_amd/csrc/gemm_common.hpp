@@ -161,7 +161,7 @@ __device__ __forceinline__ TileCoord xcd_tile_order_balanced(int mtiles, int nti
 // LDS slice `cw` (row stride CS elements) and streams it out row by row with 16-byte stores.
 // Row r of the block is output row out_row0 + r; rows at or past rows_end and columns at or past
 // N are dropped.
-template <int WM, int WNO, int CS>
+template <int WM, int WNO, int CS, bool kStream = false>
 __device__ __forceinline__ void store_wave_block(const uint16_t* __restrict__ cw, int lane, uint16_t* __restrict__ out,
                                                  int N, size_t out_row0, int rows_end, int col0) {
   constexpr int CPR_OUT = WNO / 8;
@@ -172,7 +172,13 @@ __device__ __forceinline__ void store_wave_block(const uint16_t* __restrict__ cw
     const int r = c / CPR_OUT, ch = c - r * CPR_OUT;
     const u32x4_t v = *reinterpret_cast<const u32x4_t*>(cw + r * CS + ch * 8);
     const int col = col0 + ch * 8;
-    if (r < rows_end && col < N) *reinterpret_cast<u32x4_t*>(out + (out_row0 + r) * N + col) = v;
+    if (r < rows_end && col < N) {
+      u32x4_t* const dst = reinterpret_cast<u32x4_t*>(out + (out_row0 + r) * N + col);
+      if (kStream)
+        __builtin_nontemporal_store(v, dst);  // the result is not read again by this kernel
+      else
+        *dst = v;
+    }
   }
 }
 

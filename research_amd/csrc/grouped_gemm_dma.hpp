@@ -75,7 +75,7 @@ struct DmaGemmCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NSTAGE = NSTAGE_;
   // scheduling options: 16 = request the fragments of MFMA step kk+1 before issuing step kk,
   // 32 = raise the wave priority around the MFMA burst, 64 = ask the scheduler to interleave
-  // one MFMA with up to three LDS reads
+  // one MFMA with up to three LDS reads, 128 = B tiles in 4 x 64 blocks, 32768 = non-temporal stores of the result
   static constexpr int OPT = OPT_;
   static constexpr bool kDual = kDual_;
   static constexpr int BNE = kDual ? 2 * BN : BN;  // columns of the B tile in LDS
@@ -336,7 +336,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
       }
     }
     uint16_t* const out = pass == 0 ? C : (pass == 1 ? save0 : save1);
-    store_wave_block<WM, WNO, CS>(cw, lane, out, N, (size_t)tr.row0 + row_base, tr.rows - row_base, col0);
+    store_wave_block<WM, WNO, CS, (Cfg::OPT & 32768) != 0>(cw, lane, out, N, (size_t)tr.row0 + row_base,
+                                                          tr.rows - row_base, col0);
   }
 }
 
@@ -344,7 +345,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
 // tile: 128 + 128 columns), 64-deep k steps, two LDS stages, 8 waves, B tiles in 4 x 64 blocks
 // (whole 128-byte lines per eight lanes; about 1 % faster than 4 x 16 blocks at 131072 rows).
 using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
-using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128>;
+using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128 + 32768>;  // 537 MB of results at C3: streamed out
 // Few rows per group (decode-sized batches): the layer streams every expert matrix once and
 // is bound by HBM, so the tiles are only 64 rows tall to keep the padded-row MFMA work below
 // the time the weights take to arrive, and the k steps 32 deep so that four workgroups of four

@@ -487,6 +487,22 @@ int main(int argc, char** argv) {
     ok &= check<DownNarrowCfg>("down ragged, 4 x 16 blocks", p);
     release(p);
   }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_stores")) {
+    // plain against non-temporal stores of the result, alternating on one problem
+    using GateUpNt = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128 + 32768>;
+    using DownPlain = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128>;
+    Problem g = make(64, 131072, 2048, 1408, 4, false, 0, 1.0f);
+    Problem d = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
+    ok &= check<GateUpNt>("gate/up non-temporal stores", g);
+    ok &= check<DownPlain>("down plain stores", d);
+    for (int rep = 0; rep < 3; ++rep) {
+      timeit<GateUpCfg>("gate/up plain stores (library)", g, 20);
+      timeit<GateUpNt>("gate/up non-temporal stores", g, 20);
+      timeit<DownPlain>("down plain stores", d, 20);
+      timeit<DownCfg>("down non-temporal stores (library)", d, 20);
+    }
+    release(g); release(d);
+  }
   if (ok && argc > 1 && !strcmp(argv[1], "time_backward")) time_backward();
   if (ok && argc > 1 && !strcmp(argv[1], "time_decode")) time_decode();
   if (ok && argc > 1 && !strcmp(argv[1], "time")) {
