@@ -194,7 +194,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
         const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
         cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj][i]);
       }
-  store_wave_block<WM, WN, CS>(cw, lane, C, N, (size_t)tr.row0 + wm * WM, tr.rows - wm * WM, n0 + wn * WN);
+  store_wave_block<WM, WN, CS, (Cfg::OPT & 32768) != 0>(cw, lane, C, N, (size_t)tr.row0 + wm * WM, tr.rows - wm * WM,
+                                                       n0 + wn * WN);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -441,17 +442,17 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
           cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj + which * (TN / 2)][i]);
         }
     uint16_t* const Cm = (which ? C1 : C0) + (size_t)e * KA * N;
-    store_wave_block<WM, WNO, CS>(cw, lane, Cm, N, (size_t)row_base, KA - row_base, col0);
+    store_wave_block<WM, WNO, CS, (Cfg::OPT & 32768) != 0>(cw, lane, Cm, N, (size_t)row_base, KA - row_base, col0);
     // the staging area is private to the wave and the second matrix is written by the same
     // lanes' LDS stores after their loads above: program order within the wave suffices
   }
 }
 
 // Configurations the library launches.
-using DgradCfg = NtGemmCfg<256, 256, 2, 4, 16 + 64>;   // data gradients: 256 x 256 tiles
+using DgradCfg = NtGemmCfg<256, 256, 2, 4, 16 + 64 + 32768>;   // data gradients: 256 x 256 tiles
 // narrow LDS blocks: the fastest layout when the operands are streamed (1.52 vs 1.60 ms for the
 // gate/up product of the C3 shape); the wide blocks pay off only when rows are gathered
-using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16>;  // gate and up weight gradients share the x tile
-using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16>;     // down weight gradient
+using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16 + 32768>;  // gate and up weight gradients share the x tile
+using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16 + 32768>;     // down weight gradient
 
 }  // namespace jtmoe

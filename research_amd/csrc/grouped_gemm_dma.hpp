@@ -336,8 +336,12 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
       }
     }
     uint16_t* const out = pass == 0 ? C : (pass == 1 ? save0 : save1);
-    store_wave_block<WM, WNO, CS, (Cfg::OPT & 32768) != 0>(cw, lane, out, N, (size_t)tr.row0 + row_base,
-                                                          tr.rows - row_base, col0);
+    // the kept products are read again only by the backward pass: always streamed out
+    if (pass == 0)
+      store_wave_block<WM, WNO, CS, (Cfg::OPT & 32768) != 0>(cw, lane, out, N, (size_t)tr.row0 + row_base,
+                                                            tr.rows - row_base, col0);
+    else
+      store_wave_block<WM, WNO, CS, true>(cw, lane, out, N, (size_t)tr.row0 + row_base, tr.rows - row_base, col0);
   }
 }
 
