@@ -184,6 +184,10 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
 // Mean rows per group below which the 64-row tiles are used.
 constexpr int64_t kSmallGroupRows = 128;
 inline bool small_groups(int64_t rows, int64_t E) { return rows < kSmallGroupRows * E; }
+// Mean rows per group up to which nearly every group is a single tile tall, so that no workgroup
+// reads an expert matrix after another has: its loads are then marked non-temporal.
+constexpr int64_t kTinyGroupRows = 32;
+inline bool tiny_groups(int64_t rows, int64_t E) { return rows <= kTinyGroupRows * E; }
 
 inline bool fast_ok(const void* a, const void* b0, const void* b1, const void* c, int64_t Kdim, int64_t N) {
   return Kdim % 64 == 0 && N % 8 == 0 && Kdim * N < ((int64_t)1 << 30) && aligned16(a) && aligned16(b0) && (b1 == nullptr || aligned16(b1)) &&
@@ -197,22 +201,25 @@ int launch_pair(const void* x, const void* gate, const void* up, const void* dow
                 int64_t x_rows = 0, void* save_gate = nullptr, void* save_up = nullptr) {
   if (rows == 0) return JTMOE_OK;
   int rc;
-  const bool small = small_groups(rows, E);
+  const bool small = small_groups(rows, E), tiny = tiny_groups(rows, E);
   const bool gather_ok = row_map == nullptr || x_rows * H < ((int64_t)1 << 30);
   const bool saves_ok = save_gate == nullptr || (aligned16(save_gate) && aligned16(save_up));
   if (Elem<T>::is_bf16 && fast_ok(x, gate, up, act, H, I) && gather_ok && saves_ok)
-    rc = small ? launch_fast<GateUpSmallCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
-                                             row_div, x_rows, save_gate, save_up)
-               : launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
-                                        row_div, x_rows, save_gate, save_up);
+    rc = tiny    ? launch_fast<GateUpTinyCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
+                                              row_div, x_rows, save_gate, save_up)
+         : small ? launch_fast<GateUpSmallCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
+                                               row_div, x_rows, save_gate, save_up)
+                 : launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
+                                          row_div, x_rows, save_gate, save_up);
   else
     rc = launch_generic<T, true>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map, row_div,
                                  save_gate, save_up);
   if (rc) return rc;
   stage_mark(first_stage, stream);
   if (Elem<T>::is_bf16 && fast_ok(act, down, nullptr, y, I, H))
-    rc = small ? launch_fast<DownSmallCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream)
-               : launch_fast<DownCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
+    rc = tiny    ? launch_fast<DownTinyCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream)
+         : small ? launch_fast<DownSmallCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream)
+                 : launch_fast<DownCfg>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
   else
     rc = launch_generic<T, false>(act, down, nullptr, y, group_sizes, offsets, rows, I, H, E, stream);
   if (rc) return rc;

@@ -47,6 +47,15 @@ __device__ __forceinline__ void buffer_load_lds16(i32x4_t rsrc, unsigned lds_bas
                : "memory");
 }
 
+// The same with the non-temporal hint, for operands no other workgroup reads again (the expert
+// matrices when every group is a single tile tall).
+__device__ __forceinline__ void buffer_load_lds16_nt(i32x4_t rsrc, unsigned lds_base, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+               :
+               : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+               : "memory");
+}
+
 // fp32 -> bf16 by the hardware conversion (round to nearest even)
 __device__ __forceinline__ uint16_t bf16_bits_fast(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 __device__ __forceinline__ float bf16_round_fast(float f) { return (float)(__bf16)f; }
@@ -75,7 +84,7 @@ struct DmaGemmCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NSTAGE = NSTAGE_;
   // scheduling options: 16 = request the fragments of MFMA step kk+1 before issuing step kk,
   // 32 = raise the wave priority around the MFMA burst, 64 = ask the scheduler to interleave
-  // one MFMA with up to three LDS reads, 128 = B tiles in 4 x 64 blocks, 32768 = non-temporal stores of the result
+  // one MFMA with up to three LDS reads, 128 = B tiles in 4 x 64 blocks, 4096 = non-temporal loads of B, 32768 = non-temporal stores of the result
   static constexpr int OPT = OPT_;
   static constexpr bool kDual = kDual_;
   static constexpr int BNE = kDual ? 2 * BN : BN;  // columns of the B tile in LDS
@@ -194,9 +203,14 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
 #pragma unroll
     for (int u = 0; u < Cfg::NSUB; ++u)
 #pragma unroll
-      for (int j = 0; j < Cfg::BSUB_LOADS; ++j)
-        buffer_load_lds16(b_rsrc[u], base + Cfg::A_BYTES + u * Cfg::BSUB_BYTES + j * NT * 16,
-                          b_voff[u] + j * (NT / 16) * N * 2, k0 * N * 2);
+      for (int j = 0; j < Cfg::BSUB_LOADS; ++j) {
+        if (Cfg::OPT & 4096)
+          buffer_load_lds16_nt(b_rsrc[u], base + Cfg::A_BYTES + u * Cfg::BSUB_BYTES + j * NT * 16,
+                               b_voff[u] + j * (NT / 16) * N * 2, k0 * N * 2);
+        else
+          buffer_load_lds16(b_rsrc[u], base + Cfg::A_BYTES + u * Cfg::BSUB_BYTES + j * NT * 16,
+                            b_voff[u] + j * (NT / 16) * N * 2, k0 * N * 2);
+      }
   };
 
   f32x16_t acc[TM][TN];
@@ -358,5 +372,10 @@ using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128 + 32768>;
 // last third of the workgroups ran alone on a mostly idle memory system: 0.140 vs 0.126 ms).
 using GateUpSmallCfg = DmaGemmCfg<64, 128, 32, 1, 4, true, 2, 16 + 128>;
 using DownSmallCfg = DmaGemmCfg<64, 256, 32, 1, 4, false, 2, 16>;
+// The same tiles when nearly every group fits one tile (a decode step): each expert matrix is then
+// read by exactly one row of workgroups, and non-temporal loads stream it past the L2
+// (64 tokens, 64 experts: gate/up 0.126 -> 0.110 ms = 6.7 TB/s, down 0.061 -> 0.054 ms = 6.8 TB/s).
+using GateUpTinyCfg = DmaGemmCfg<64, 128, 32, 1, 4, true, 2, 16 + 128 + 4096>;
+using DownTinyCfg = DmaGemmCfg<64, 256, 32, 1, 4, false, 2, 16 + 4096>;
 
 }  // namespace jtmoe

@@ -417,12 +417,16 @@ static void time_backward() {
 // decode-sized batch: 8 rows per group, bound by streaming the expert matrices
 static void time_decode() {
   Problem g = make(64, 512, 2048, 1408, 8, false, 0, 1.0f);
-  timeit<GateUpCfg>("gate/up 64 groups, 256-row tiles", g, 20);
-  timeit<GateUpSmallCfg>("gate/up 64 groups, 64-row tiles", g, 20);
-  release(g);
   Problem d = make(64, 512, 1408, 2048, 9, false, 0, 1.0f);
+  timeit<GateUpCfg>("gate/up 64 groups, 256-row tiles", g, 20);
   timeit<DownCfg>("down 64 groups, 256-row tiles", d, 20);
-  timeit<DownSmallCfg>("down 64 groups, 64-row tiles", d, 20);
+  for (int rep = 0; rep < 3; ++rep) {
+    timeit<GateUpSmallCfg>("gate/up 64 groups, 64-row tiles", g, 50);
+    timeit<GateUpTinyCfg>("gate/up 64 groups, 64-row tiles, weights non-temporal", g, 50);
+    timeit<DownSmallCfg>("down 64 groups, 64-row tiles", d, 50);
+    timeit<DownTinyCfg>("down 64 groups, 64-row tiles, weights non-temporal", d, 50);
+  }
+  release(g);
   release(d);
 }
 
@@ -454,7 +458,12 @@ int main(int argc, char** argv) {
   {
     Problem p = make(5, 300, 512, 384, 7, true, 3, 1.0f);
     ok &= check<GateUpSmallCfg>("gate/up few rows, gather on load", p);
+    ok &= check<GateUpTinyCfg>("gate/up few rows, gather, streamed weights", p);
     release(p);
+    Problem q = make(16, 150, 512, 392, 8, true, 0, 1.0f);
+    ok &= check<GateUpTinyCfg>("gate/up few rows, streamed weights", q);
+    ok &= check<DownTinyCfg>("down few rows, streamed weights", q);
+    release(q);
   }
   {
     Problem p = make(7, 3001, 576, 392, 11, true, 0, 1.0f);
