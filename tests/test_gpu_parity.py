@@ -203,7 +203,9 @@ def random_problem(seed, tokens, hidden, experts, top_k, inter, std=0.2):
     "tokens,hidden,experts,top_k,inter,dtype",
     [(8, 3, 4, 2, 5, "f32"), (70, 32, 4, 2, 64, "f32"), (200, 512, 8, 2, 1024, "f32"),
      (8, 3, 4, 2, 5, "bf16"), (300, 64, 6, 3, 96, "bf16"), (700, 1024, 16, 2, 2816, "bf16"),
-     (512, 2048, 64, 8, 1408, "bf16"), (64, 2048, 64, 8, 1408, "bf16"), (257, 200, 5, 2, 136, "bf16")],
+     (512, 2048, 64, 8, 1408, "bf16"), (64, 2048, 64, 8, 1408, "bf16"), (257, 200, 5, 2, 136, "bf16"),
+     # either side of the mean of 32 rows per group up to which the expert matrices are streamed
+     (128, 1024, 8, 2, 704, "bf16"), (129, 1024, 8, 2, 704, "bf16")],
 )
 def test_grouped_swiglu_matches_oracle(gpu, tokens, hidden, experts, top_k, inter, dtype):
     std = 0.02 if hidden >= 512 else 0.2
