@@ -68,3 +68,35 @@ def test_random_expert_and_combine_shapes(gpu, seed):
         top_k = int(rng.choice([1, 2, 3, 8]))
         print(f"combine {dtype} T={tokens} H={hidden} K={top_k}", flush=True)
         P.test_combine_is_bit_exact(gpu, tokens, hidden, top_k, dtype, bool(rng.random() < 0.5))
+
+
+@pytest.mark.parametrize("seed", [41])
+def test_random_gradient_shapes(gpu, seed):
+    """The backward operators on odd shapes: rows that leave the fast GEMM paths, single tokens,
+    one expert, top_k = num_experts."""
+    import test_gpu_grad as G
+
+    rng = np.random.default_rng(seed)
+    for _ in range(10):
+        tokens = int(rng.choice([1, 5, 40, 130, 300]))
+        hidden = int(rng.choice([8, 24, 64, 200, 512]))
+        experts = int(rng.choice([1, 2, 5, 8, 16]))
+        top_k = int(rng.integers(1, min(experts, 4) + 1))
+        inter = int(rng.choice([8, 40, 64, 136, 256]))
+        dtype = "f32" if hidden <= 64 and inter <= 64 and rng.random() < 0.5 else "bf16"
+        print(f"expert gradients {dtype} T={tokens} H={hidden} E={experts} K={top_k} I={inter}", flush=True)
+        G.test_expert_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, inter, dtype)
+    for _ in range(6):
+        tokens, hidden, inter = int(rng.choice([1, 7, 64, 300])), int(rng.choice([8, 72, 256, 1024])), int(rng.choice([8, 40, 704]))
+        # fp32 only where the sums are short: the element-wise fp32 bar of that check is tighter than the
+        # difference between two summation orders over hundreds of terms
+        dtype = "f32" if hidden <= 72 and inter <= 40 and rng.random() < 0.5 else "bf16"
+        print(f"shared gradients {dtype} T={tokens} H={hidden} I={inter}", flush=True)
+        G.test_shared_gradients_match_oracle(gpu, tokens, hidden, inter, dtype)
+    for _ in range(8):
+        dtype = "bf16" if rng.random() < 0.7 else "f32"
+        tokens, hidden = int(rng.choice([1, 9, 64, 257, 600])), int(rng.choice([8, 72, 256, 1024]))
+        experts = int(rng.choice([1, 3, 8, 24, 64, 256]))
+        top_k = int(rng.integers(1, min(experts, 8) + 1))
+        print(f"router gradients {dtype} T={tokens} H={hidden} E={experts} K={top_k}", flush=True)
+        G.test_router_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, dtype, bool(rng.random() < 0.5))
