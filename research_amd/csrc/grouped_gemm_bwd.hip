@@ -199,6 +199,31 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
   out[i] = (uint16_t)f32_to_bf16_bits(acc);
 }
 
+// four elements per thread; the partial sums are read once
+typedef float stream_f32x4_t __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void reduce_partials_vec_kernel(const stream_f32x4_t* __restrict__ partial,
+                                                                  int splits, size_t nvec, uint2* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  stream_f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int s = 0; s < splits; ++s) {
+    const stream_f32x4_t v = __builtin_nontemporal_load(&partial[(size_t)s * nvec + i]);
+    acc += v;
+  }
+  out[i] = make_uint2(f32_to_bf16_bits(acc[0]) | (f32_to_bf16_bits(acc[1]) << 16),
+                      f32_to_bf16_bits(acc[2]) | (f32_to_bf16_bits(acc[3]) << 16));
+}
+
+void launch_reduce_partials(const float* partial, int splits, size_t n, uint16_t* out, hipStream_t stream) {
+  if (n % 4 == 0 && aligned16(partial) && (reinterpret_cast<uintptr_t>(out) & 7) == 0) {
+    const size_t nvec = n / 4;
+    reduce_partials_vec_kernel<<<(unsigned)((nvec + 255) / 256), 256, 0, stream>>>(
+        reinterpret_cast<const stream_f32x4_t*>(partial), splits, nvec, reinterpret_cast<uint2*>(out));
+  } else {
+    reduce_partials_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(partial, splits, n, out);
+  }
+}
+
 struct SplitPlan {
   int splits;  // 0: do not split
   int chunk;   // rows per run, a multiple of the k step
@@ -243,9 +268,8 @@ int launch_tn_fast(const void* p, const void* d0, const void* d1, void* c0, void
         static_cast<const uint16_t*>(p), static_cast<const uint16_t*>(d0), static_cast<const uint16_t*>(d1),
         reinterpret_cast<uint16_t*>(part0), reinterpret_cast<uint16_t*>(part1), nullptr, nullptr, plan.splits,
         (int)rows, (int)KA, (int)N, (int)mt, (int)nt, nullptr, 1, 0, 0, 0, plan.chunk);
-    const unsigned rgrid = (unsigned)((n + 255) / 256);
-    reduce_partials_kernel<<<rgrid, 256, 0, stream>>>(part0, plan.splits, n, static_cast<uint16_t*>(c0));
-    if (Cfg::kDual) reduce_partials_kernel<<<rgrid, 256, 0, stream>>>(part1, plan.splits, n, static_cast<uint16_t*>(c1));
+    launch_reduce_partials(part0, plan.splits, n, static_cast<uint16_t*>(c0), stream);
+    if (Cfg::kDual) launch_reduce_partials(part1, plan.splits, n, static_cast<uint16_t*>(c1), stream);
     return JTMOE_OK;
   }
   const int64_t grid = gemm_grid(E * mt, nt);
