@@ -119,15 +119,24 @@ static void release(Problem& p) {
   hipFree(p.dgs); hipFree(p.doff); hipFree(p.drow); hipFree(p.darow); hipFree(p.dmap);
 }
 
+// The 256-row configurations run as the library runs them: persistent workgroups, one per CU (256
+// here), unless g_one_tile_per_workgroup asks for the plain kernel.
+static bool g_one_tile_per_workgroup = false;
 template <typename Cfg>
 static void launch(Problem& p, bool dense) {
+  constexpr bool kCanPersist = Cfg::BM == 256 && Cfg::NSTAGE == 2 && Cfg::BK == 64;
+  const bool persist = kCanPersist && !g_one_tile_per_workgroup;
   auto kernel = grouped_gemm_dma_kernel<Cfg>;
+  if constexpr (kCanPersist) {
+    if (persist) kernel = grouped_gemm_dma_persistent_kernel<Cfg>;
+  }
   CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                          (int)Cfg::SMEM_BYTES));
   const long mt = dense ? (p.rows + Cfg::BM - 1) / Cfg::BM
                         : (p.rows + Cfg::BM - 1) / Cfg::BM + (p.E < p.rows ? p.E : p.rows);
   const long nt = (p.N + Cfg::BN - 1) / Cfg::BN;
-  kernel<<<(unsigned)gemm_grid(mt, nt), Cfg::NT, Cfg::SMEM_BYTES>>>(
+  const long tiles_grid = gemm_grid(mt, nt);
+  kernel<<<(unsigned)(persist && tiles_grid > 256 ? 256 : tiles_grid), Cfg::NT, Cfg::SMEM_BYTES>>>(
       p.A, p.B0, Cfg::kDual ? p.B1 : nullptr, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows,
       p.K, p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, nullptr, nullptr);
 }
@@ -495,6 +504,39 @@ int main(int argc, char** argv) {
     ok &= check<GateUpNarrowCfg>("gate/up ragged, 4 x 16 blocks", p);
     ok &= check<DownNarrowCfg>("down ragged, 4 x 16 blocks", p);
     release(p);
+  }
+  {
+    // the one-tile-per-workgroup kernel with the 256-row configurations (the library runs them persistently)
+    g_one_tile_per_workgroup = true;
+    Problem p = make(7, 3001, 576, 392, 24, true, 0, 1.0f);
+    ok &= check<GateUpCfg>("gate/up ragged, one tile per workgroup", p);
+    ok &= check<DownCfg>("down ragged, one tile per workgroup", p);
+    release(p);
+    Problem q = make(5, 2400, 512, 384, 25, true, 3, 1.0f);
+    ok &= check<GateUpCfg>("gate/up gather, one tile per workgroup", q);
+    release(q);
+    g_one_tile_per_workgroup = false;
+    Problem t = make(3, 700, 64, 136, 26, false, 0, 1.0f);  // a single k step per tile
+    ok &= check<GateUpCfg>("gate/up one k step", t);
+    ok &= check<DownCfg>("down one k step", t);
+    release(t);
+    Problem u = make(40, 70000, 128, 264, 27, true, 0, 1.0f);  // many more tiles than workgroups
+    ok &= check<GateUpCfg>("gate/up many tiles per workgroup", u);
+    ok &= check<DownCfg>("down many tiles per workgroup", u);
+    release(u);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_persistent")) {
+    Problem g = make(64, 131072, 2048, 1408, 4, false, 0, 1.0f);
+    Problem d = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
+    for (int rep = 0; rep < 3; ++rep) {
+      g_one_tile_per_workgroup = true;
+      timeit<GateUpCfg>("gate/up one tile per workgroup", g, 20);
+      timeit<DownCfg>("down one tile per workgroup", d, 20);
+      g_one_tile_per_workgroup = false;
+      timeit<GateUpCfg>("gate/up persistent (library)", g, 20);
+      timeit<DownCfg>("down persistent (library)", d, 20);
+    }
+    release(g); release(d);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_stores")) {
     // plain against non-temporal stores of the result, alternating on one problem
