@@ -185,4 +185,17 @@ __device__ __forceinline__ void store_wave_block(const uint16_t* __restrict__ cw
 // number of workgroups for `mtiles x ntiles_n` tiles: a multiple of 8 (one slice per XCD)
 inline int64_t gemm_grid(int64_t mtiles, int64_t ntiles_n) { return (mtiles * ntiles_n + 7) / 8 * 8; }
 
+// number of workgroups of a persistent launch: one per CU of the current device, a whole number per
+// XCD (the 256-row configurations fit one workgroup per CU); looked up once per process
+inline int persistent_grid_size() {
+  static const int size = [] {
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus < 8)
+      return 8;
+    return cus / 8 * 8;
+  }();
+  return size;
+}
+
 }  // namespace jtmoe

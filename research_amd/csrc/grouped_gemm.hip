@@ -163,7 +163,6 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   constexpr bool kPersistent = Cfg::BM == 256 && Cfg::NSTAGE == 2 && Cfg::BK == 64;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  static int persistent_grid = 0;
   auto kernel = [] {
     if constexpr (kPersistent)
       return &grouped_gemm_dma_persistent_kernel<Cfg>;
@@ -173,10 +172,6 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)Cfg::SMEM_BYTES);
-    int device = 0, cus = 0;
-    if (attr_err == hipSuccess) attr_err = hipGetDevice(&device);
-    if (attr_err == hipSuccess) attr_err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
-    persistent_grid = cus >= 8 ? cus / 8 * 8 : 8;  // one workgroup per CU, a whole number per XCD
   });
   if (attr_err != hipSuccess)
     return fail(JTMOE_ELAUNCH, "grouped gemm: kernel set-up: %s", hipGetErrorString(attr_err));
@@ -185,7 +180,7 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   const int64_t nt = (N + Cfg::BN - 1) / Cfg::BN;
   const int64_t tiles_grid = gemm_grid(mtiles, nt);
   if (tiles_grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
-  const int64_t grid = kPersistent && tiles_grid > persistent_grid ? persistent_grid : tiles_grid;
+  const int64_t grid = kPersistent && tiles_grid > persistent_grid_size() ? persistent_grid_size() : tiles_grid;
   kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
       static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
       static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,

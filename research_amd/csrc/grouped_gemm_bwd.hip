@@ -163,8 +163,10 @@ int launch_gemm_nt(int dtype, const void* a0, const void* a1, const void* b0, co
       return fail(JTMOE_ELAUNCH, "grouped gemm (nt): hipFuncSetAttribute: %s", hipGetErrorString(attr_err));
     const int64_t mtiles = dense ? (rows + Cfg::BM - 1) / Cfg::BM : max_m_tiles(rows, E, Cfg::BM);
     const int64_t nt = (N + Cfg::BN - 1) / Cfg::BN;
-    const int64_t grid = gemm_grid(mtiles, nt);
-    if (grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm (nt): grid too large");
+    const int64_t tiles_grid = gemm_grid(mtiles, nt);
+    if (tiles_grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm (nt): grid too large");
+    // persistent workgroups: one per CU, each walking its share of the tiles
+    const int64_t grid = tiles_grid > persistent_grid_size() ? persistent_grid_size() : tiles_grid;
     kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
         static_cast<const uint16_t*>(a0), static_cast<const uint16_t*>(a1), static_cast<const uint16_t*>(b0),
         static_cast<const uint16_t*>(b1), static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows,

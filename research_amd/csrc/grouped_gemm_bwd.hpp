@@ -58,58 +58,87 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
-  // the grid covers an upper bound of the m-tiles; the tile order is cut from their real number
-  TileCoord tc;
-  TileRows tr;
-  if (group_sizes) {
-    const GroupScan scan = group_scan(BM, group_sizes, E);
-    tc = xcd_tile_order_balanced(scan.total, ntiles_n, Cfg::GROUP_M);
-    if (tc.mt < 0) return;
-    tr = locate_tile(scan, tc.mt, BM, offsets);
-  } else {
-    tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
-    if (tc.mt < 0) return;
-    tr = find_tile_wave(tc.mt, BM, nullptr, nullptr, E, dense_rows);
-  }
-  const int nt = tc.nt;
-  tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
-  tr.row0 = __builtin_amdgcn_readfirstlane(tr.row0);
-  tr.rows = __builtin_amdgcn_readfirstlane(tr.rows);
-  if (tr.rows <= 0) return;
-  const int n0 = nt * BN;
-  const size_t wofs = (size_t)tr.expert * Kdim * N;
-
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WAVES_N, wn = wave - wm * Cfg::WAVES_N;
-
   const bool gather = row_map != nullptr;
-  i32x4_t a_rsrc[2], b_rsrc[2];
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const uint16_t* a = s ? A1 : A0;
-    const uint16_t* b = s ? B1 : B0;
-    if (s >= segs) {
-      a = A0;
-      b = B0;
-    }
-    a_rsrc[s] = gather ? make_rsrc(a, a_rows * Kdim * 2) : make_rsrc(a + (size_t)tr.row0 * Kdim, tr.rows * Kdim * 2);
-    // rows of B past N lie outside the descriptor and read as zeros
-    b_rsrc[s] = make_rsrc(b + wofs, N * Kdim * 2);
+
+  // Persistent workgroups, as in grouped_gemm_dma_persistent_kernel: this one walks the tiles
+  // idx, idx + stride, ... of its XCD's contiguous range of the logical order.
+  GroupScan scan;
+  int real_mtiles = mtiles;
+  if (group_sizes) {
+    scan = group_scan(BM, group_sizes, E);
+    real_mtiles = __builtin_amdgcn_readfirstlane(scan.total);
   }
+  const int total = real_mtiles * ntiles_n;
+  const int per_xcd = (total + 7) >> 3;
+  const int xcd = (int)blockIdx.x & 7, stride = max(1, (int)gridDim.x >> 3);
+  int idx = (int)blockIdx.x >> 3;
+  struct Tile {
+    int expert, row0, rows, n0;
+  };
+  auto locate = [&](int i) -> Tile {
+    Tile t;
+    t.expert = 0; t.row0 = 0; t.rows = 0; t.n0 = 0;
+    const int logical = xcd * per_xcd + i;
+    if (i >= per_xcd || logical >= total) return t;
+    const int group_span = Cfg::GROUP_M * ntiles_n;
+    const int group = logical / group_span;
+    const int in_group = logical - group * group_span;
+    const int gm = min(Cfg::GROUP_M, real_mtiles - group * Cfg::GROUP_M);
+    const int nt = in_group / gm;
+    const int mt = group * Cfg::GROUP_M + (in_group - nt * gm);
+    TileRows tr;
+    if (group_sizes) {
+      tr = locate_tile(scan, mt, BM, offsets);
+    } else {
+      tr.expert = 0;
+      tr.row0 = mt * BM;
+      tr.rows = min(BM, dense_rows - mt * BM);
+    }
+    t.expert = __builtin_amdgcn_readfirstlane(tr.expert);
+    t.row0 = __builtin_amdgcn_readfirstlane(tr.row0);
+    t.rows = __builtin_amdgcn_readfirstlane(tr.rows);
+    t.n0 = nt * BN;
+    return t;
+  };
+
+  // ---- load plan (rewritten for every tile) ----
+  i32x4_t a_rsrc[2], b_rsrc[2];
   // both tiles: slot s = j*NT + tid -> row s/8, slot-in-row s%8 holds source chunk (s%8) ^ ((row/2)%8)
   const int l_r = tid >> 3, l_slot = tid & 7;
   const int l_c = l_slot ^ ((l_r >> 1) & 7);
   int a_voff[Cfg::A_LOADS];
+  int b_voff = 0;
+  auto row_offsets = [&](const Tile& t, int* voff) {
 #pragma unroll
-  for (int j = 0; j < Cfg::A_LOADS; ++j) {
-    const int r = l_r + j * (NT / 8);
-    if (gather)
-      a_voff[j] = r < tr.rows ? ((row_map[tr.row0 + r] / row_div) * Kdim + l_c * 8) * 2 : 0x70000000;
-    else
-      a_voff[j] = (r * Kdim + l_c * 8) * 2;
-  }
-  const int b_voff = ((n0 + l_r) * Kdim + l_c * 8) * 2;
+    for (int j = 0; j < Cfg::A_LOADS; ++j) {
+      const int r = l_r + j * (NT / 8);
+      if (gather)
+        voff[j] = r < t.rows ? ((row_map[t.row0 + r] / row_div) * Kdim + l_c * 8) * 2 : 0x70000000;
+      else
+        voff[j] = (r * Kdim + l_c * 8) * 2;
+    }
+  };
+  auto plan = [&](const Tile& t, const int* voff) {
+    const size_t wofs = (size_t)t.expert * Kdim * N;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const uint16_t* a = s ? A1 : A0;
+      const uint16_t* b = s ? B1 : B0;
+      if (s >= segs) {
+        a = A0;
+        b = B0;
+      }
+      a_rsrc[s] = gather ? make_rsrc(a, a_rows * Kdim * 2) : make_rsrc(a + (size_t)t.row0 * Kdim, t.rows * Kdim * 2);
+      // rows of B past N lie outside the descriptor and read as zeros
+      b_rsrc[s] = make_rsrc(b + wofs, N * Kdim * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < Cfg::A_LOADS; ++j) a_voff[j] = voff[j];
+    b_voff = ((t.n0 + l_r) * Kdim + l_c * 8) * 2;
+  };
   const unsigned lds0 = lds_byte_addr(smem_raw);
   const unsigned wave_lds = lds0 + wave * 1024;
   const int nk1 = Kdim / BK;
@@ -128,14 +157,6 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
       buffer_load_lds16(br, base + Cfg::A_BYTES + j * NT * 16, b_voff + j * (NT / 8) * Kdim * 2, k0 * 2);
   };
 
-  f32x16_t acc[TM][TN];
-#pragma unroll
-  for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-    for (int jj = 0; jj < TN; ++jj)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
-
   const int sw = ((lane & 31) >> 1) & 7;
   const int a_rowoff = (wm * WM + (lane & 31)) * (BK * 2);
   const int b_rowoff = Cfg::A_BYTES + (wn * WN + (lane & 31)) * (BK * 2);
@@ -150,52 +171,91 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
       bf[jj] = *reinterpret_cast<const bf16x8_t*>(st + b_rowoff + jj * 32 * BK * 2 + chunk);
   };
 
-  // a wave whose rows all lie past the end of the group skips its fragment reads and MFMAs
-  const bool wave_has_rows = wm * WM < tr.rows;
-  if (nk > 0) issue(0);
-  for (int kt = 0; kt < nk; ++kt) {
-    wait_vmcnt<0>();
-    __syncthreads();
-    if (kt + 1 < nk) issue(kt + 1);
-    if (!wave_has_rows) continue;
-    const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
-    bf16x8_t af[2][TM], bf[2][TN];
-    load_frags(st, 0, af[0], bf[0]);
+  // Epilogue staging lives above the first stage buffer, which the next tile's first loads fill
+  // while the epilogue runs; a wave's block goes out in halves where it does not fit its share.
+  constexpr int CS = Cfg::CS;
+  constexpr int kStageArea = (int)Cfg::SMEM_BYTES - Cfg::STAGE_BYTES;
+  constexpr int kHalves = (NT / 64) * WM * CS * 2 <= kStageArea ? 1 : 2;
+  constexpr int TMH = TM / kHalves, WMH = WM / kHalves;
+  static_assert((NT / 64) * WMH * CS * 2 <= kStageArea && TM % kHalves == 0, "epilogue staging must fit above stage 0");
+  uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw + Cfg::STAGE_BYTES) + wave * (WMH * CS);
+
+  Tile cur = locate(idx);
+  if (cur.rows <= 0 || nk <= 0) return;
+  {
+    int voff[Cfg::A_LOADS];
+    row_offsets(cur, voff);
+    plan(cur, voff);
+  }
+  issue(0);
+
+  while (true) {
+    f32x16_t acc[TM][TN];
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+    for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
-      for (int mi = 0; mi < TM; ++mi)
+      for (int jj = 0; jj < TN; ++jj)
 #pragma unroll
-        for (int jj = 0; jj < TN; ++jj)
-          acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
-      if (Cfg::OPT & 64) {
+        for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
+    // a wave whose rows all lie past the end of the group skips its fragment reads and MFMAs
+    const bool wave_has_rows = wm * WM < cur.rows;
+    // the tile after this one is looked up now, and its row offsets requested
+    idx += stride;
+    const Tile nxt = locate(idx);
+    int nxt_voff[Cfg::A_LOADS];
+    if (nxt.rows > 0) row_offsets(nxt, nxt_voff);
+
+    for (int kt = 0; kt < nk; ++kt) {
+      wait_vmcnt<0>();
+      __syncthreads();
+      if (kt + 1 < nk) issue(kt + 1);
+      if (!wave_has_rows) continue;
+      const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
+      bf16x8_t af[2][TM], bf[2][TN];
+      load_frags(st, 0, af[0], bf[0]);
 #pragma unroll
-        for (int g = 0; g < TM * TN; ++g) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+          for (int jj = 0; jj < TN; ++jj)
+            acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
+        if (Cfg::OPT & 64) {
+#pragma unroll
+          for (int g = 0; g < TM * TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+          }
         }
       }
     }
-  }
-  wait_vmcnt<0>();
-  __syncthreads();
+    __syncthreads();  // every wave is done reading the stage buffers
 
-  // epilogue: each wave parks its WM x WN block in its own slice of the idle LDS and streams it
-  // out row by row with 16-byte stores
-  constexpr int CS = Cfg::CS;
-  uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
+    // the first operand tiles of the next tile are on their way while this one's results go out
+    const int out_row0 = cur.row0, out_rows = cur.rows, out_n0 = cur.n0;
+    if (nxt.rows > 0) {
+      plan(nxt, nxt_voff);
+      issue(0);
+    }
 #pragma unroll
-  for (int mi = 0; mi < TM; ++mi)
+    for (int h = 0; h < kHalves; ++h) {
+      const int row_base = wm * WM + h * WMH;
 #pragma unroll
-    for (int jj = 0; jj < TN; ++jj)
+      for (int mh = 0; mh < TMH; ++mh)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-        cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj][i]);
-      }
-  store_wave_block<WM, WN, CS, (Cfg::OPT & 32768) != 0>(cw, lane, C, N, (size_t)tr.row0 + wm * WM, tr.rows - wm * WM,
-                                                       n0 + wn * WN);
+        for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int r = mh * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+            cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[h * TMH + mh][jj][i]);
+          }
+      store_wave_block<WMH, WN, CS, (Cfg::OPT & 32768) != 0>(cw, lane, C, N, (size_t)out_row0 + row_base,
+                                                            out_rows - row_base, out_n0 + wn * WN);
+    }
+    if (nxt.rows <= 0) break;
+    cur = nxt;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -255,7 +255,9 @@ static void launch_nt(Problem& p, const uint16_t* A1, int segs, bool dense) {
   const long mt = dense ? (p.rows + Cfg::BM - 1) / Cfg::BM
                         : (p.rows + Cfg::BM - 1) / Cfg::BM + (p.E < p.rows ? p.E : p.rows);
   const long nt = (p.N + Cfg::BN - 1) / Cfg::BN;
-  kernel<<<(unsigned)gemm_grid(mt, nt), Cfg::NT, Cfg::SMEM_BYTES>>>(
+  // persistent workgroups, as the library launches it; g_one_tile_per_workgroup gives every tile its own
+  const long tiles_grid = gemm_grid(mt, nt);
+  kernel<<<(unsigned)(!g_one_tile_per_workgroup && tiles_grid > 256 ? 256 : tiles_grid), Cfg::NT, Cfg::SMEM_BYTES>>>(
       p.A, A1, p.B0, p.B1, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows, p.K, p.N, (int)mt,
       (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, segs);
 }
@@ -524,6 +526,31 @@ int main(int argc, char** argv) {
     ok &= check<GateUpCfg>("gate/up many tiles per workgroup", u);
     ok &= check<DownCfg>("down many tiles per workgroup", u);
     release(u);
+  }
+  {
+    Problem u = make(40, 70000, 128, 264, 28, true, 0, 1.0f);  // many more tiles than workgroups
+    ok &= check_nt<DgradCfg>("dgrad many tiles per workgroup", u, 1);
+    ok &= check_nt<DgradCfg>("dgrad many tiles per workgroup, two segments", u, 2);
+    release(u);
+    Problem v = make(9, 20000, 64, 520, 29, true, 3, 1.0f);  // one k step, gathered rows
+    ok &= check_nt<DgradCfg>("dgrad one k step, gather on load", v, 1);
+    release(v);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_persistent_nt")) {
+    const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
+    Problem p = make(E, rows, H, I, 21, false, 0, 1.0f);   // Z = dYp @ Wd^T
+    Problem q = make(E, rows, I, H, 22, false, 0, 1.0f);   // dXp = dG @ Wg^T + dU @ Wu^T
+    uint16_t* A1 = random_bf16((size_t)rows * I, 33, 1.0f);
+    for (int rep = 0; rep < 3; ++rep) {
+      g_one_tile_per_workgroup = true;
+      time_launches("dgrad down, one tile per workgroup", 2.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(p, nullptr, 1, false); });
+      time_launches("dgrad gate/up, one tile per workgroup", 4.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(q, A1, 2, false); });
+      g_one_tile_per_workgroup = false;
+      time_launches("dgrad down, persistent (library)", 2.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(p, nullptr, 1, false); });
+      time_launches("dgrad gate/up, persistent (library)", 4.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(q, A1, 2, false); });
+    }
+    hipFree(A1);
+    release(p); release(q);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_persistent")) {
     Problem g = make(64, 131072, 2048, 1408, 4, false, 0, 1.0f);
