@@ -265,7 +265,8 @@ int launch_tn_fast(const void* p, const void* d0, const void* d1, void* c0, void
     const size_t n = (size_t)KA * N;
     float* part0 = static_cast<float*>(split_ws);
     float* part1 = part0 + (size_t)plan.splits * n;
-    const int64_t grid = gemm_grid(plan.splits * mt, nt);
+    const int64_t tiles_grid = gemm_grid(plan.splits * mt, nt);
+    const int64_t grid = tiles_grid > persistent_grid_size() ? persistent_grid_size() : tiles_grid;
     kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
         static_cast<const uint16_t*>(p), static_cast<const uint16_t*>(d0), static_cast<const uint16_t*>(d1),
         reinterpret_cast<uint16_t*>(part0), reinterpret_cast<uint16_t*>(part1), nullptr, nullptr, plan.splits,
@@ -274,8 +275,10 @@ int launch_tn_fast(const void* p, const void* d0, const void* d1, void* c0, void
     if (Cfg::kDual) launch_reduce_partials(part1, plan.splits, n, static_cast<uint16_t*>(c1), stream);
     return JTMOE_OK;
   }
-  const int64_t grid = gemm_grid(E * mt, nt);
-  if (grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm (tn): grid too large");
+  const int64_t tiles_grid = gemm_grid(E * mt, nt);
+  if (tiles_grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm (tn): grid too large");
+  // persistent workgroups: one per CU, each walking its share of the (group, tile) pairs
+  const int64_t grid = tiles_grid > persistent_grid_size() ? persistent_grid_size() : tiles_grid;
   kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
       static_cast<const uint16_t*>(p), static_cast<const uint16_t*>(d0), static_cast<const uint16_t*>(d1),
       static_cast<uint16_t*>(c0), static_cast<uint16_t*>(c1), group_sizes, offsets, (int)E, (int)rows, (int)KA,

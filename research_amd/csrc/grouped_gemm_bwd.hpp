@@ -300,46 +300,53 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   constexpr bool kDual = Cfg::kDual;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
-  // consecutive workgroup ids go round-robin to the 8 XCDs: give each XCD a contiguous range of
-  // (group, tile) pairs so that all tiles of one group read its rows through the same L2
-  const int per_group = mtiles_o * ntiles_o;
-  const int total = E * per_group;
-  const int per_xcd = (int)gridDim.x >> 3;
-  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
-  if (logical >= total) return;
-  const int e = logical / per_group;
-  const int in_e = logical - e * per_group;
-  const int nt = in_e / mtiles_o;
-  const int mt = in_e - nt * mtiles_o;
-  const int m0 = mt * BMO, n0 = nt * BNO;
-
-  // split_chunk > 0 (one dense group only): "group" e is the e-th run of split_chunk rows, and the
-  // outputs are float32 partial sums [E, KA, N] that the caller adds up in a fixed order.  This
-  // gives a reduction over many rows into a small matrix enough workgroups to fill the chip.
-  int row0, rows;
-  if (group_sizes) {
-    row0 = __builtin_amdgcn_readfirstlane(offsets[e]);
-    rows = __builtin_amdgcn_readfirstlane(group_sizes[e]);
-  } else if (split_chunk > 0) {
-    row0 = e * split_chunk;
-    rows = max(0, min(split_chunk, dense_rows - row0));
-  } else {
-    row0 = 0;
-    rows = dense_rows;
-  }
-
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WAVES_N, wn = wave - wm * Cfg::WAVES_N;
 
-  const i32x4_t p_rsrc = p_gather ? make_rsrc(P, gathered_rows * KA * 2)
-                                  : make_rsrc(P + (size_t)row0 * KA, rows * KA * 2);
+  // Persistent workgroups: consecutive workgroup ids go round-robin to the 8 XCDs, each XCD owns a
+  // contiguous range of (group, tile) pairs (so that all tiles of one group read its rows through
+  // the same L2), and this workgroup walks the pairs idx, idx + stride, ... of its XCD's range.
+  const int per_group = mtiles_o * ntiles_o;
+  const int total = E * per_group;
+  const int per_xcd = (total + 7) >> 3;
+  const int xcd = (int)blockIdx.x & 7, stride = max(1, (int)gridDim.x >> 3);
+  int idx = (int)blockIdx.x >> 3;
+
+  // split_chunk > 0 (one dense group only): "group" e is the e-th run of split_chunk rows, and the
+  // outputs are float32 partial sums [E, KA, N] that the caller adds up in a fixed order.  This
+  // gives a reduction over many rows into a small matrix enough workgroups to fill the chip.
+  struct Tile {
+    int e, m0, n0, row0, rows;
+    bool valid;
+  };
+  auto locate = [&](int i) -> Tile {
+    Tile t;
+    t.e = 0; t.m0 = 0; t.n0 = 0; t.row0 = 0; t.rows = 0;
+    const int logical = xcd * per_xcd + i;
+    t.valid = i < per_xcd && logical < total;
+    if (!t.valid) return t;
+    t.e = logical / per_group;
+    const int in_e = logical - t.e * per_group;
+    const int nt = in_e / mtiles_o;
+    t.m0 = (in_e - nt * mtiles_o) * BMO;
+    t.n0 = nt * BNO;
+    if (group_sizes) {
+      t.row0 = __builtin_amdgcn_readfirstlane(offsets[t.e]);
+      t.rows = __builtin_amdgcn_readfirstlane(group_sizes[t.e]);
+    } else if (split_chunk > 0) {
+      t.row0 = t.e * split_chunk;
+      t.rows = max(0, min(split_chunk, dense_rows - t.row0));
+    } else {
+      t.row0 = 0;
+      t.rows = dense_rows;
+    }
+    return t;
+  };
+
+  // ---- load plan (rewritten for every tile) ----
+  i32x4_t p_rsrc;
   i32x4_t d_rsrc[Cfg::DSUB];
-#pragma unroll
-  for (int u = 0; u < Cfg::DSUB; ++u) {
-    const uint16_t* d = (kDual && u == 1) ? D1 : D0;
-    d_rsrc[u] = d_gather ? make_rsrc(d, gathered_rows * N * 2) : make_rsrc(d + (size_t)row0 * N, rows * N * 2);
-  }
   // sub-tile [BK rows][128 columns] as 128-byte blocks of 4 rows x 16 columns, block (r/4, c/16) at
   // index (r/4)*8 + c/16; slot s (16 bytes) -> block s/8, row (s/2)%4 of the block, half s%2
   // (OPT & 128: 512-byte blocks of 4 rows x 64 columns instead, block (r/4, c/64) at index
@@ -352,10 +359,23 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   // puts the four 32-byte pieces of a transposing read into four different groups of banks)
   const int l_c = kWide ? (b_blk_id & 1) * 8 + ((tid & 7) ^ (((tid >> 4) & 1) << 2)) : (b_blk_id & 7) * 2 + (tid & 1);
   constexpr int ROWS_PER_LOAD = NT / 16;
-  const int p_col = (m0 + l_c * 8) * 2, d_col = (n0 + l_c * 8) * 2;  // byte offset inside a row
+  int p_col = 0, d_col = 0;  // byte offset inside a row
+  int row0 = 0, rows = 0, nk = 0;
+  auto plan = [&](const Tile& t) {
+    row0 = t.row0;
+    rows = t.rows;
+    nk = (rows + BK - 1) / BK;
+    p_rsrc = p_gather ? make_rsrc(P, gathered_rows * KA * 2) : make_rsrc(P + (size_t)row0 * KA, rows * KA * 2);
+#pragma unroll
+    for (int u = 0; u < Cfg::DSUB; ++u) {
+      const uint16_t* d = (kDual && u == 1) ? D1 : D0;
+      d_rsrc[u] = d_gather ? make_rsrc(d, gathered_rows * N * 2) : make_rsrc(d + (size_t)row0 * N, rows * N * 2);
+    }
+    p_col = (t.m0 + l_c * 8) * 2;
+    d_col = (t.n0 + l_c * 8) * 2;
+  };
   const unsigned lds0 = lds_byte_addr(smem_raw);
   const unsigned wave_lds = lds0 + wave * 1024;
-  const int nk = (rows + BK - 1) / BK;
 
   // row ids of a k step (only used by gathered operands); -1 = past the end of the group
   int ids[Cfg::SUB_LOADS];
@@ -367,7 +387,6 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
     }
   };
   const bool any_gather = p_gather || d_gather;
-  if (any_gather && nk > 0) fetch_ids(0);
 
   // Rows past the end of the group must contribute zeros: their offsets lie outside the
   // descriptor (which ends with the group, or is pushed there explicitly for gathered rows).
@@ -380,26 +399,31 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
       pv[j] = p_gather ? (ids[j] >= 0 ? ids[j] * KA * 2 + p_col : 0x70000000) : r * KA * 2 + p_col;
       dv[j] = d_gather ? (ids[j] >= 0 ? ids[j] * N * 2 + d_col : 0x70000000) : r * N * 2 + d_col;
     }
-#pragma unroll
-    for (int u = 0; u < Cfg::PSUB; ++u)
-#pragma unroll
-      for (int j = 0; j < Cfg::SUB_LOADS; ++j)
-        buffer_load_lds16(p_rsrc, base + u * Cfg::SUB_BYTES + j * NT * 16, pv[j] + u * 256, 0);
-#pragma unroll
-    for (int u = 0; u < Cfg::DSUB; ++u)
-#pragma unroll
-      for (int j = 0; j < Cfg::SUB_LOADS; ++j)
-        buffer_load_lds16(d_rsrc[u], base + Cfg::P_BYTES + u * Cfg::SUB_BYTES + j * NT * 16,
-                          dv[j] + (kDual ? 0 : u * 256), 0);
+    // LDS address = one scalar per stage + a compile-time offset per load (this kernel is short of
+    // scalar registers)
+    static_assert(Cfg::PSUB <= 2 && Cfg::DSUB <= 2 && Cfg::SUB_LOADS == 2, "load list written out below");
+    buffer_load_lds16_at<0>(p_rsrc, base, pv[0], 0);
+    buffer_load_lds16_at<NT * 16>(p_rsrc, base, pv[1], 0);
+    if (Cfg::PSUB == 2) {
+      buffer_load_lds16_at<Cfg::SUB_BYTES>(p_rsrc, base, pv[0] + 256, 0);
+      buffer_load_lds16_at<Cfg::SUB_BYTES + NT * 16>(p_rsrc, base, pv[1] + 256, 0);
+    }
+    buffer_load_lds16_at<Cfg::P_BYTES>(d_rsrc[0], base, dv[0], 0);
+    buffer_load_lds16_at<Cfg::P_BYTES + NT * 16>(d_rsrc[0], base, dv[1], 0);
+    if (Cfg::DSUB == 2) {
+      buffer_load_lds16_at<Cfg::P_BYTES + Cfg::SUB_BYTES>(d_rsrc[Cfg::DSUB - 1], base, dv[0] + (kDual ? 0 : 256), 0);
+      buffer_load_lds16_at<Cfg::P_BYTES + Cfg::SUB_BYTES + NT * 16>(d_rsrc[Cfg::DSUB - 1], base,
+                                                                  dv[1] + (kDual ? 0 : 256), 0);
+    }
   };
-
-  f32x16_t acc[TM][TN];
-#pragma unroll
-  for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-    for (int jj = 0; jj < TN; ++jj)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
+  // first loads of a tile (and, for gathered operands, the row ids they need)
+  auto start_tile = [&]() {
+    if (nk > 0) {
+      if (any_gather) fetch_ids(0);
+      issue(0);
+      if (any_gather && nk > 1) fetch_ids(1);
+    }
+  };
 
   // transposing read: the 16 lanes of a group read one whole 128-byte block, lane i its bytes
   // [8 i, 8 i + 8) = row i/4, columns 4*(i%4)..; groups: column half (lane/16)%2, row half lane/32
@@ -438,73 +462,107 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
     for (int jj = 0; jj < TN; ++jj) bf[jj] = read_tr(st + d_blk[jj] + laneoff + kk * (4 * 8 * 128));
   };
 
-  if (nk > 0) {
-    issue(0);
-    if (any_gather && nk > 1) fetch_ids(1);
-  }
-  for (int kt = 0; kt < nk; ++kt) {
-    wait_vmcnt<0>();
-    __syncthreads();
-    if (kt + 1 < nk) {
-      issue(kt + 1);
-      if (any_gather && kt + 2 < nk) fetch_ids(kt + 2);
-    }
-    const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
-    bf16x8_t af[2][TM], bf[2][TN];
-    load_frags(st, 0, af[0], bf[0]);
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-#pragma unroll
-      for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-        for (int jj = 0; jj < TN; ++jj)
-          acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
-    }
-  }
-  wait_vmcnt<0>();
-  __syncthreads();
-
+  // Epilogue staging lives above the first stage buffer, which the next tile's first loads fill
+  // while the epilogue runs; a wave's block goes out in halves where it does not fit its share.
   constexpr int TNO = Cfg::TNO, WNO = Cfg::WNO, CS = Cfg::CS;
-  if (split_chunk > 0) {
-    // float32 partial sums straight from the accumulators: for a fixed i the 32 lanes of a half
-    // wave write 128 contiguous bytes of one row
-#pragma unroll
-    for (int which = 0; which < (kDual ? 2 : 1); ++which) {
-      float* const Cm = reinterpret_cast<float*>(which ? C1 : C0) + (size_t)e * KA * N;
-#pragma unroll
-      for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-        for (int jj = 0; jj < TNO; ++jj) {
-          const int col = n0 + wn * WNO + jj * 32 + (lane & 31);
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int r = m0 + wm * WM + mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-            if (r < KA && col < N) Cm[(size_t)r * N + col] = acc[mi][jj + which * (TN / 2)][i];
-          }
-        }
-    }
-    return;
-  }
-  // epilogue: per matrix, each wave parks its WM x WNO block in LDS and streams it out in rows
-  uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw) + wave * (WM * CS);
-  const int col0 = n0 + wn * WNO;
-  const int row_base = m0 + wm * WM;
-#pragma unroll
-  for (int which = 0; which < (kDual ? 2 : 1); ++which) {
+  constexpr int kStageArea = (int)Cfg::SMEM_BYTES - Cfg::STAGE_BYTES;
+  constexpr int kHalves = (NT / 64) * WM * CS * 2 <= kStageArea ? 1 : 2;
+  constexpr int TMH = TM / kHalves, WMH = WM / kHalves;
+  static_assert((NT / 64) * WMH * CS * 2 <= kStageArea && TM % kHalves == 0, "epilogue staging must fit above stage 0");
+  uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw + Cfg::STAGE_BYTES) + wave * (WMH * CS);
+
+  Tile cur = locate(idx);
+  if (!cur.valid) return;
+  plan(cur);
+  start_tile();
+
+  while (true) {
+    f32x16_t acc[TM][TN];
 #pragma unroll
     for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
-      for (int jj = 0; jj < TNO; ++jj)
+      for (int jj = 0; jj < TN; ++jj)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int r = mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-          cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[mi][jj + which * (TN / 2)][i]);
+        for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
+
+    for (int kt = 0; kt < nk; ++kt) {
+      wait_vmcnt<0>();
+      __syncthreads();
+      if (kt + 1 < nk) {
+        issue(kt + 1);
+        if (any_gather && kt + 2 < nk) fetch_ids(kt + 2);
+      }
+      const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
+      bf16x8_t af[2][TM], bf[2][TN];
+      load_frags(st, 0, af[0], bf[0]);
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+          for (int jj = 0; jj < TN; ++jj)
+            acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
+      }
+    }
+    __syncthreads();  // every wave is done reading the stage buffers (and, for an empty group, with
+                      // the previous tile's staging area)
+
+    // the first operand tiles of the next pair are on their way while this one's results go out
+    // (the pair is looked up only now: this kernel has no scalar registers to spare during the k loop)
+    const int out_e = cur.e, out_m0 = cur.m0, out_n0 = cur.n0;
+    idx += stride;
+    const Tile nxt = locate(idx);
+    if (nxt.valid) {
+      plan(nxt);
+      start_tile();
+    }
+
+    if (split_chunk > 0) {
+      // float32 partial sums straight from the accumulators: for a fixed i the 32 lanes of a half
+      // wave write 128 contiguous bytes of one row
+#pragma unroll
+      for (int which = 0; which < (kDual ? 2 : 1); ++which) {
+        float* const Cm = reinterpret_cast<float*>(which ? C1 : C0) + (size_t)out_e * KA * N;
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+          for (int jj = 0; jj < TNO; ++jj) {
+            const int col = out_n0 + wn * WNO + jj * 32 + (lane & 31);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int r = out_m0 + wm * WM + mi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+              if (r < KA && col < N) Cm[(size_t)r * N + col] = acc[mi][jj + which * (TN / 2)][i];
+            }
+          }
+      }
+    } else {
+      // per matrix, each wave parks its block in LDS (in halves) and streams it out in rows
+      const int col0 = out_n0 + wn * WNO;
+#pragma unroll
+      for (int which = 0; which < (kDual ? 2 : 1); ++which) {
+        uint16_t* const Cm = (which ? C1 : C0) + (size_t)out_e * KA * N;
+#pragma unroll
+        for (int h = 0; h < kHalves; ++h) {
+          const int row_base = out_m0 + wm * WM + h * WMH;
+#pragma unroll
+          for (int mh = 0; mh < TMH; ++mh)
+#pragma unroll
+            for (int jj = 0; jj < TNO; ++jj)
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                const int r = mh * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+                cw[r * CS + jj * 32 + (lane & 31)] = bf16_bits_fast(acc[h * TMH + mh][jj + which * (TN / 2)][i]);
+              }
+          // the staging area is private to the wave: program order within the wave suffices between
+          // one block's row stores and the next block's LDS writes
+          store_wave_block<WMH, WNO, CS, (Cfg::OPT & 32768) != 0>(cw, lane, Cm, N, (size_t)row_base, KA - row_base,
+                                                                 col0);
         }
-    uint16_t* const Cm = (which ? C1 : C0) + (size_t)e * KA * N;
-    store_wave_block<WM, WNO, CS, (Cfg::OPT & 32768) != 0>(cw, lane, Cm, N, (size_t)row_base, KA - row_base, col0);
-    // the staging area is private to the wave and the second matrix is written by the same
-    // lanes' LDS stores after their loads above: program order within the wave suffices
+      }
+    }
+    if (!nxt.valid) break;
+    cur = nxt;
   }
 }
 

@@ -47,6 +47,16 @@ __device__ __forceinline__ void buffer_load_lds16(i32x4_t rsrc, unsigned lds_bas
                : "memory");
 }
 
+// The same with the LDS address given as a scalar base plus a compile-time offset: a kernel that
+// issues many loads per stage then keeps one scalar per stage instead of one per load.
+template <int kOffset>
+__device__ __forceinline__ void buffer_load_lds16_at(i32x4_t rsrc, unsigned lds_base, int voffset, int soffset) {
+  asm volatile("s_add_u32 m0, %0, %4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset), "n"(kOffset)
+               : "memory", "scc");
+}
+
 // The same with the non-temporal hint, for operands no other workgroup reads again (the expert
 // matrices when every group is a single tile tall).
 __device__ __forceinline__ void buffer_load_lds16_nt(i32x4_t rsrc, unsigned lds_base, int voffset, int soffset) {

@@ -289,7 +289,8 @@ static void launch_tn(Problem& p, const uint16_t* D0, const uint16_t* D1, uint16
                          (int)Cfg::SMEM_BYTES));
   const long mt = (p.K + Cfg::BMO - 1) / Cfg::BMO, nt = (p.N + Cfg::BNO - 1) / Cfg::BNO;
   const int groups = dense ? 1 : p.E;
-  kernel<<<(unsigned)gemm_grid(groups * mt, nt), Cfg::NT, Cfg::SMEM_BYTES>>>(
+  const long tiles_grid = gemm_grid(groups * mt, nt);
+  kernel<<<(unsigned)(!g_one_tile_per_workgroup && tiles_grid > 256 ? 256 : tiles_grid), Cfg::NT, Cfg::SMEM_BYTES>>>(
       p.A, D0, D1, C0, C1, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, groups, p.rows, p.K, p.N, (int)mt,
       (int)nt, p.dmap, p.top_k > 0 ? p.top_k : 1, p_gather, d_gather, p.a_rows, 0);
 }
@@ -535,6 +536,36 @@ int main(int argc, char** argv) {
     Problem v = make(9, 20000, 64, 520, 29, true, 3, 1.0f);  // one k step, gathered rows
     ok &= check_nt<DgradCfg>("dgrad one k step, gather on load", v, 1);
     release(v);
+  }
+  {
+    Problem u = make(40, 30000, 520, 264, 30, true, 0, 1.0f);  // many more (group, tile) pairs than workgroups
+    ok &= check_tn<WgradCfg>("wgrad many pairs per workgroup", u, 0);
+    ok &= check_tn<WgradDualCfg>("wgrad dual many pairs per workgroup", u, 0);
+    release(u);
+    Problem v = make(70, 20000, 520, 264, 31, true, 3, 1.0f);  // the same with gathered operands and empty groups
+    ok &= check_tn<WgradDualCfg>("wgrad dual many pairs, transposed operand gathered", v, 1);
+    ok &= check_tn<WgradCfg>("wgrad many pairs, other operand gathered", v, 2);
+    release(v);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_persistent_tn")) {
+    const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
+    Problem p = make(E, rows, H, I, 21, false, 0, 1.0f);
+    uint16_t* D0 = random_bf16((size_t)rows * I, 31, 1.0f);
+    uint16_t* D1 = random_bf16((size_t)rows * I, 32, 1.0f);
+    uint16_t *C0, *C1;
+    CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
+    Problem q = make(E, rows, I, H, 23, false, 0, 1.0f);
+    uint16_t* dYp = random_bf16((size_t)rows * H, 37, 1.0f);
+    for (int rep = 0; rep < 3; ++rep) {
+      g_one_tile_per_workgroup = true;
+      time_launches("wgrad gate/up, one pair per workgroup", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad down, one pair per workgroup", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+      g_one_tile_per_workgroup = false;
+      time_launches("wgrad gate/up, persistent (library)", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad down, persistent (library)", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+    }
+    hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
+    release(p); release(q);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_persistent_nt")) {
     const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
