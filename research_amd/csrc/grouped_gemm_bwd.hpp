@@ -307,11 +307,54 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   // Persistent workgroups: consecutive workgroup ids go round-robin to the 8 XCDs, each XCD owns a
   // contiguous range of (group, tile) pairs (so that all tiles of one group read its rows through
   // the same L2), and this workgroup walks the pairs idx, idx + stride, ... of its XCD's range.
+  // A pair's k loop is as long as its group, so with groups of unequal sizes the ranges are cut
+  // by work (k steps plus a fixed cost per pair), not by the number of pairs.
   const int per_group = mtiles_o * ntiles_o;
   const int total = E * per_group;
-  const int per_xcd = (total + 7) >> 3;
   const int xcd = (int)blockIdx.x & 7, stride = max(1, (int)gridDim.x >> 3);
   int idx = (int)blockIdx.x >> 3;
+  int pair_lo = min(total, xcd * ((total + 7) >> 3)), pair_hi = min(total, (xcd + 1) * ((total + 7) >> 3));
+  if (group_sizes) {
+    constexpr int kPer = JTMOE_MAX_EXPERTS / 64;  // groups per lane, contiguous
+    constexpr int kFixedSteps = 3;                // look-up and epilogue of a pair, in k steps
+    int w[kPer], local = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int e = lane * kPer + j;
+      w[j] = e < E ? (group_sizes[e] + BK - 1) / BK + kFixedSteps : 0;
+      local += w[j];
+    }
+    int incl = local;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int v = __shfl_up(incl, d);
+      if (lane >= d) incl += v;
+    }
+    const long long first = (long long)(incl - local) * per_group;  // work before this lane's groups
+    const long long all = (long long)__shfl(incl, 63) * per_group;
+    // the first pair that starts at or after `target` units of work
+    auto first_pair_at = [&](long long target) -> int {
+      const bool mine = target >= first && target < first + (long long)local * per_group;
+      const unsigned long long owners = __ballot(mine);
+      if (owners == 0ull) return total;  // target == all
+      const int owner = __ffsll((long long)owners) - 1;
+      int pair = 0;
+      long long s = first;
+      bool found = false;
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const long long span = (long long)w[j] * per_group;
+        if (mine && !found && target < s + span) {
+          pair = (lane * kPer + j) * per_group + ((int)(target - s) + w[j] - 1) / w[j];
+          found = true;
+        }
+        s += span;
+      }
+      return __builtin_amdgcn_readfirstlane(__shfl(pair, owner));
+    };
+    pair_lo = first_pair_at(all * xcd / 8);
+    pair_hi = first_pair_at(all * (xcd + 1) / 8);
+  }
 
   // split_chunk > 0 (one dense group only): "group" e is the e-th run of split_chunk rows, and the
   // outputs are float32 partial sums [E, KA, N] that the caller adds up in a fixed order.  This
@@ -323,8 +366,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   auto locate = [&](int i) -> Tile {
     Tile t;
     t.e = 0; t.m0 = 0; t.n0 = 0; t.row0 = 0; t.rows = 0;
-    const int logical = xcd * per_xcd + i;
-    t.valid = i < per_xcd && logical < total;
+    const int logical = pair_lo + i;
+    t.valid = logical < pair_hi;
     if (!t.valid) return t;
     t.e = logical / per_group;
     const int in_e = logical - t.e * per_group;

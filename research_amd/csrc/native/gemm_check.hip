@@ -546,6 +546,30 @@ int main(int argc, char** argv) {
     ok &= check_tn<WgradDualCfg>("wgrad dual many pairs, transposed operand gathered", v, 1);
     ok &= check_tn<WgradCfg>("wgrad many pairs, other operand gathered", v, 2);
     release(v);
+    Problem w = make(256, 50000, 136, 264, 32, true, 0, 1.0f);  // the most groups, very unequal sizes
+    ok &= check_tn<WgradCfg>("wgrad 256 unequal groups", w, 0);
+    ok &= check_tn<WgradDualCfg>("wgrad dual 256 unequal groups", w, 0);
+    release(w);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_unequal_tn")) {
+    // weight gradients over groups of very unequal sizes (128 groups, 131072 rows)
+    const int E = 128, rows = 131072, H = 2048, I = 768;
+    Problem p = make(E, rows, H, I, 41, true, 0, 1.0f);
+    int longest = 0;
+    for (int n : p.gs) longest = std::max(longest, n);
+    printf("longest group: %d rows of %d\n", longest, rows);
+    uint16_t* D0 = random_bf16((size_t)rows * I, 42, 1.0f);
+    uint16_t* D1 = random_bf16((size_t)rows * I, 43, 1.0f);
+    uint16_t *C0, *C1;
+    CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
+    Problem q = make(E, rows, I, H, 41, true, 0, 1.0f);
+    uint16_t* dYp = random_bf16((size_t)rows * H, 44, 1.0f);
+    for (int rep = 0; rep < 3; ++rep) {
+      time_launches("wgrad gate/up, unequal groups", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad down, unequal groups", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+    }
+    hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
+    release(p); release(q);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_persistent_tn")) {
     const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
