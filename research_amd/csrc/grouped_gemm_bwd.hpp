@@ -198,7 +198,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
     // a wave whose rows all lie past the end of the group skips its fragment reads and MFMAs
-    const bool wave_has_rows = wm * WM < cur.rows;
+    // a wave whose rows lie past the end of the group, or whose columns lie past N, has nothing to add
+    const bool wave_has_rows = wm * WM < cur.rows && cur.n0 + wn * WN < N;
     // the tile after this one is looked up now, and its row offsets requested
     idx += stride;
     const Tile nxt = locate(idx);
@@ -528,6 +529,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
 
+    // a wave whose block of the result lies wholly outside [KA, N] has nothing to add
+    const bool wave_has_output = cur.m0 + wm * WM < KA && cur.n0 + wn * (kDual ? WN / 2 : WN) < N;
     for (int kt = 0; kt < nk; ++kt) {
       wait_vmcnt<0>();
       __syncthreads();
@@ -535,6 +538,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
         issue(kt + 1);
         if (any_gather && kt + 2 < nk) fetch_ids(kt + 2);
       }
+      if (!wave_has_output) continue;
       const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
       bf16x8_t af[2][TM], bf[2][TN];
       load_frags(st, 0, af[0], bf[0]);

@@ -274,8 +274,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
 
   const int nk = Kdim / BK;
   // The last tile of a group is usually partly empty.  A wave whose WM rows all lie past the end of
-  // the group still takes part in the loads and the barriers but skips its fragment reads and MFMAs.
-  const bool wave_has_rows = wm * WM < tr.rows;
+  // the group (or whose columns all lie past N) still takes part in the loads and the barriers but
+  // skips its fragment reads and MFMAs.
+  const bool wave_has_rows = wm * WM < tr.rows && n0 + wn * Cfg::WNO < N;
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s)
     if (s < nk) issue(s);
@@ -553,7 +554,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
       for (int jj = 0; jj < TN; ++jj)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
-    const bool wave_has_rows = wm * WM < cur.rows;
+    const bool wave_has_rows = wm * WM < cur.rows && cur.n0 + wn * Cfg::WNO < N;
     // the tile after this one is looked up now, and its row offsets requested, so that nothing but the
     // issue of its first loads stands between the end of this tile's k loop and its epilogue
     idx += stride;
