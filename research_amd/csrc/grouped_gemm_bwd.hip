@@ -5,6 +5,7 @@
 #include "gemm_launch.hpp"
 #include "grouped_gemm_bwd.hpp"
 
+#include <algorithm>
 #include <mutex>
 
 namespace jtmoe {
@@ -231,17 +232,36 @@ struct SplitPlan {
   int chunk;   // rows per run, a multiple of the k step
 };
 
-// A one-group reduction is split when its output tiles cannot occupy the chip and there are
-// enough rows to share out.
+// A one-group reduction whose output tiles cannot occupy the chip is split into runs of rows.
+// The number of runs minimises an estimate of the launch in k steps: rounds of (tile, run) pairs over
+// the CUs times the steps of a run (plus a fixed cost per pair), plus the reduction of the float32
+// partial sums (written and read once per run: about 0.8 steps per million result elements).  A
+// split is taken only when it is estimated to save a tenth of the time.
 template <typename Cfg>
 SplitPlan split_plan(int64_t rows, int64_t KA, int64_t N) {
   const int64_t tiles = ((KA + Cfg::BMO - 1) / Cfg::BMO) * ((N + Cfg::BNO - 1) / Cfg::BNO);
   SplitPlan p{0, 0};
-  if (tiles > 128 || rows < 2048) return p;
-  int64_t splits = (512 + tiles - 1) / tiles;
-  if (splits > rows / 256) splits = rows / 256;
-  if (splits < 2) return p;
-  const int64_t chunk = ((rows + splits - 1) / splits + 63) / 64 * 64;
+  const int64_t cus = persistent_grid_size();
+  if (tiles > cus || rows < 2048) return p;
+  const double reduce_steps = 0.84e-6 * (double)KA * (double)N * (Cfg::kDual ? 2.0 : 1.0);
+  auto cost = [&](int64_t runs) {
+    const int64_t chunk = ((rows + runs - 1) / runs + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
+    const int64_t real_runs = (rows + chunk - 1) / chunk;
+    const int64_t rounds = (tiles * real_runs + cus - 1) / cus;
+    return (double)rounds * (double)(chunk / Cfg::BK + 3) + (real_runs > 1 ? reduce_steps * (double)real_runs : 0.0);
+  };
+  const int64_t max_runs = std::min<int64_t>(64, rows / 256);
+  int64_t best = 1;
+  double best_cost = cost(1);
+  for (int64_t runs = 2; runs <= max_runs; ++runs) {
+    const double c = cost(runs);
+    if (c < best_cost) {
+      best_cost = c;
+      best = runs;
+    }
+  }
+  if (best < 2 || best_cost > 0.9 * cost(1)) return p;
+  const int64_t chunk = ((rows + best - 1) / best + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
   p.splits = (int)((rows + chunk - 1) / chunk);
   p.chunk = (int)chunk;
   return p;
