@@ -307,29 +307,47 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
 
   // Persistent workgroups: consecutive workgroup ids go round-robin to the 8 XCDs, each XCD owns a
   // contiguous range of (group, tile) pairs (so that all tiles of one group read its rows through
-  // the same L2), and this workgroup walks the pairs idx, idx + stride, ... of its XCD's range.
-  // A pair's k loop is as long as its group, so with groups of unequal sizes the ranges are cut
-  // by work (k steps plus a fixed cost per pair), not by the number of pairs.
+  // the same L2).  A pair's k loop is as long as its group.  With groups of about the same size
+  // the ranges hold the same number of pairs and this workgroup walks the pairs idx, idx + stride,
+  // ... of its XCD's range.  With unequal groups the ranges are cut by work (k steps plus a fixed
+  // cost per pair), and the pairs of a range are dealt longest group first, each to the workgroup
+  // with the least work so far: every workgroup of the XCD runs the same deterministic deal and
+  // keeps its own list.
   const int per_group = mtiles_o * ntiles_o;
   const int total = E * per_group;
   const int xcd = (int)blockIdx.x & 7, stride = max(1, (int)gridDim.x >> 3);
   int idx = (int)blockIdx.x >> 3;
   int pair_lo = min(total, xcd * ((total + 7) >> 3)), pair_hi = min(total, (xcd + 1) * ((total + 7) >> 3));
+  constexpr int kMaxList = 2048;  // pairs a range may hold for the deal (else: round-robin)
+  __shared__ int s_work[JTMOE_MAX_EXPERTS], s_count[JTMOE_MAX_EXPERTS], s_first[JTMOE_MAX_EXPERTS];
+  __shared__ int s_order[JTMOE_MAX_EXPERTS];
+  __shared__ int s_list[kMaxList];
+  __shared__ int s_len;
+  int listed = -1;  // >= 0: this workgroup's pairs are s_list[0 .. listed)
   if (group_sizes) {
     constexpr int kPer = JTMOE_MAX_EXPERTS / 64;  // groups per lane, contiguous
     constexpr int kFixedSteps = 3;                // look-up and epilogue of a pair, in k steps
-    int w[kPer], local = 0;
+    int w[kPer], local = 0, wmin = 0x7fffffff, wmax = 0;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int e = lane * kPer + j;
       w[j] = e < E ? (group_sizes[e] + BK - 1) / BK + kFixedSteps : 0;
       local += w[j];
+      if (e < E) {
+        wmin = min(wmin, w[j]);
+        wmax = max(wmax, w[j]);
+      }
     }
     int incl = local;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const int v = __shfl_up(incl, d);
       if (lane >= d) incl += v;
+    }
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      wmin = min(wmin, __shfl_xor(wmin, d));
+      wmax = max(wmax, __shfl_xor(wmax, d));
     }
     const long long first = (long long)(incl - local) * per_group;  // work before this lane's groups
     const long long all = (long long)__shfl(incl, 63) * per_group;
@@ -353,9 +371,77 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
       }
       return __builtin_amdgcn_readfirstlane(__shfl(pair, owner));
     };
-    pair_lo = first_pair_at(all * xcd / 8);
-    pair_hi = first_pair_at(all * (xcd + 1) / 8);
+    wmin = __builtin_amdgcn_readfirstlane(wmin);
+    wmax = __builtin_amdgcn_readfirstlane(wmax);
+    const bool unequal = (long long)wmax * 4 > (long long)wmin * 5;  // longest group > 1.25 x shortest
+    const bool keys_fit = __builtin_amdgcn_readfirstlane((int)(all < ((long long)1 << 26))) != 0;
+    if (unequal) {
+      pair_lo = first_pair_at(all * xcd / 8);
+      pair_hi = first_pair_at(all * (xcd + 1) / 8);
+    }
+    // the deal (work of one XCD must fit the 26 bits the arg-min key leaves for it)
+    if (unequal && pair_hi - pair_lo <= kMaxList && stride <= 32 && keys_fit) {
+      if (wave == 0) {
+        // groups with pairs inside the range: work, number of pairs inside, first pair inside
+        int inside = 0;
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = lane * kPer + j;
+          const int lo = max(pair_lo, e * per_group), hi = min(pair_hi, (e + 1) * per_group);
+          s_work[e] = w[j];
+          s_count[e] = e < E ? max(0, hi - lo) : 0;
+          s_first[e] = lo;
+          inside += e < E && hi > lo;
+        }
+        // (same wave: LDS writes above are visible to the reads below after the wait the compiler places)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        // order: longer groups first, equal ones by index
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = lane * kPer + j;
+          if (e < E && s_count[e] > 0) {
+            int rank = 0;
+            for (int o = 0; o < E; ++o)
+              rank += s_count[o] > 0 && (s_work[o] > w[j] || (s_work[o] == w[j] && o < e));
+            s_order[rank] = e;
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        int n_inside = inside;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) n_inside += __shfl_xor(n_inside, d);
+        n_inside = __builtin_amdgcn_readfirstlane(n_inside);
+        // lanes 0 .. stride-1 stand for the workgroups of this XCD
+        int load = lane < stride ? 0 : (1 << 26) - 1;
+        int len = 0;
+        for (int r = 0; r < n_inside; ++r) {
+          const int e = __builtin_amdgcn_readfirstlane(s_order[r]);
+          const int we = __builtin_amdgcn_readfirstlane(s_work[e]);
+          const int cnt = __builtin_amdgcn_readfirstlane(s_count[e]);
+          const int fst = __builtin_amdgcn_readfirstlane(s_first[e]);
+          for (int c = 0; c < cnt; ++c) {
+            int key = (load << 5) | (lane & 31);
+            key = min(key, __builtin_amdgcn_mov_dpp(key, 0xB1, 0xF, 0xF, false));   // lanes ^ 1
+            key = min(key, __builtin_amdgcn_mov_dpp(key, 0x4E, 0xF, 0xF, false));   // lanes ^ 2
+            key = min(key, __builtin_amdgcn_mov_dpp(key, 0x141, 0xF, 0xF, false));  // mirror within 8
+            key = min(key, __builtin_amdgcn_mov_dpp(key, 0x140, 0xF, 0xF, false));  // mirror within 16
+            const int least = min(__builtin_amdgcn_readlane(key, 0), __builtin_amdgcn_readlane(key, 16)) & 31;
+            if (lane == least) load += we;
+            if (least == idx) {
+              if (lane == 0) s_list[len] = fst + c;
+              ++len;
+            }
+          }
+        }
+        if (lane == 0) s_len = len;
+      }
+      __syncthreads();
+      listed = __builtin_amdgcn_readfirstlane(s_len);
+    }
   }
+  int step = 0;  // number of pairs this workgroup has taken
 
   // split_chunk > 0 (one dense group only): "group" e is the e-th run of split_chunk rows, and the
   // outputs are float32 partial sums [E, KA, N] that the caller adds up in a fixed order.  This
@@ -367,8 +453,14 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   auto locate = [&](int i) -> Tile {
     Tile t;
     t.e = 0; t.m0 = 0; t.n0 = 0; t.row0 = 0; t.rows = 0;
-    const int logical = pair_lo + i;
-    t.valid = logical < pair_hi;
+    int logical;
+    if (listed >= 0) {
+      t.valid = i < listed;
+      logical = t.valid ? __builtin_amdgcn_readfirstlane(s_list[i]) : 0;
+    } else {
+      logical = pair_lo + idx + i * stride;
+      t.valid = logical < pair_hi;
+    }
     if (!t.valid) return t;
     t.e = logical / per_group;
     const int in_e = logical - t.e * per_group;
@@ -515,7 +607,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   static_assert((NT / 64) * WMH * CS * 2 <= kStageArea && TM % kHalves == 0, "epilogue staging must fit above stage 0");
   uint16_t* const cw = reinterpret_cast<uint16_t*>(smem_raw + Cfg::STAGE_BYTES) + wave * (WMH * CS);
 
-  Tile cur = locate(idx);
+  Tile cur = locate(step);
   if (!cur.valid) return;
   plan(cur);
   start_tile();
@@ -558,8 +650,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
     // the first operand tiles of the next pair are on their way while this one's results go out
     // (the pair is looked up only now: this kernel has no scalar registers to spare during the k loop)
     const int out_e = cur.e, out_m0 = cur.m0, out_n0 = cur.n0;
-    idx += stride;
-    const Tile nxt = locate(idx);
+    ++step;
+    const Tile nxt = locate(step);
     if (nxt.valid) {
       plan(nxt);
       start_tile();
