@@ -92,6 +92,46 @@ def test_expert_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, inte
         assert not got.d_gate[e].any() and not got.d_up[e].any() and not got.d_down[e].any()
 
 
+@pytest.mark.parametrize("tokens,hidden,experts,top_k,inter", [(1500, 512, 64, 4, 384), (900, 1024, 40, 2, 704)])
+def test_expert_gradients_with_one_dominant_group(gpu, tokens, hidden, experts, top_k, inter):
+    """Very unequal groups: one expert takes a slot of most tokens, a third of the experts get nothing.
+
+    The weight-gradient launch then has more (group, tile) pairs than workgroups and hands them out
+    longest group first; every pair must still be computed exactly once.
+    """
+    x, gate, up, down, ids, w = random_problem(7 + tokens, tokens, hidden, experts, top_k, inter, 0.02)
+    rng = np.random.default_rng(tokens)
+    live = experts - experts // 3
+    ids = np.stack([rng.permutation(live)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    heavy = rng.random(tokens) < 0.8
+    ids[heavy, 0] = 0
+    for t in np.nonzero(heavy)[0]:  # keep the slots of a token distinct
+        dup = np.nonzero(ids[t, 1:] == 0)[0]
+        if dup.size:
+            ids[t, 1 + dup[0]] = live - 1 if live - 1 not in ids[t] else next(e for e in range(1, live) if e not in ids[t])
+    dy = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    cast = lambda a: O.cast_compute(a, "bf16")
+    want = G.experts_backward(cast(x), ids, cast(w), cast(gate), cast(up), cast(down), cast(dy))
+    got, (_, _, _, plan) = expert_grads(gpu, x, ids, w, gate, up, down, dy, "bf16")
+    again, _ = expert_grads(gpu, x, ids, w, gate, up, down, dy, "bf16")
+    sizes = host(plan.group_sizes)
+    assert sizes.max() > 10 * np.median(sizes[sizes > 0]) and (sizes == 0).sum() >= experts // 3
+    tag = f"dominant group T={tokens} H={hidden} E={experts} K={top_k} I={inter}"
+    for name in ("dx", "d_weights", "d_gate", "d_up", "d_down"):
+        ref = getattr(want, name).astype(np.float32)
+        assert report(f"{tag} {name}", host(getattr(got, name)), ref) <= BF16_MAX_REL
+        assert torch.equal(getattr(got, name), getattr(again, name)), f"{name} differs between two identical calls"
+    # per expert, so that a small expert's matrices are not hidden behind the dominant one's scale
+    for name in ("d_gate", "d_up", "d_down"):
+        g, ref = host(getattr(got, name)), getattr(want, name).astype(np.float32)
+        for e in range(experts):
+            if sizes[e] == 0:
+                assert not g[e].any()
+            else:
+                scale = float(np.max(np.abs(ref[e])))
+                assert float(np.max(np.abs(g[e] - ref[e]))) <= BF16_MAX_REL * scale, f"{tag} {name}[{e}]"
+
+
 # the 4096-token cases take the path that splits a long one-group reduction into partial sums
 @pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16"),
                                                        (4096, 512, 704, "bf16"), (64, 1024, 704, "bf16")])
