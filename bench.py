@@ -194,8 +194,8 @@ def train_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, work) -> dic
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=20)
-    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--config", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
     parser.add_argument("--cpu-sample-tokens", type=int, default=8192)
     parser.add_argument("--no-cpu-baseline", action="store_true")
