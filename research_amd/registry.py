@@ -165,6 +165,36 @@ def library_cache_status(root: str | Path | None = None) -> tuple[str, str]:
     return ("cached" if _sha256(path) == expected else "stale"), rel_path
 
 
+# Stable names of how the routed experts run, for artifacts that must not change silently between a
+# run and its resumption: the reference records `expert_execution` and `grouped_gemm_lowering` in
+# the dispatcher payload that enters its diagnostics and its resume fingerprint
+# (src/jaxtitan/models/execution.py:29-33, 136-138; src/jaxtitan/runtime/resume.py:87-97, 115).
+EXPERT_EXECUTION = "expert_major_jtmoe_grouped_gemm"
+GROUPED_GEMM_LOWERING = "hip_gfx950_lds_dma_mfma"
+
+
+def expert_execution_payload(root: str | Path | None = None) -> dict[str, Any]:
+    """The fields a run's diagnostics and resume metadata carry when this library runs the experts.
+
+    `library_sha256` is the manifest's checksum of the shared object (None unless the cache is
+    intact): two runs with the same value execute the same machine code, so a resumed run can
+    insist on it, or on the two names alone if a rebuilt library is acceptable.
+    """
+    status, _ = library_cache_status(root)
+    sha = None
+    if status == "cached":
+        manifest = load_cache_manifest(root)
+        sha = manifest["artifacts"]["moe"]["ffi"]["sha256"]
+    return {
+        "expert_execution": EXPERT_EXECUTION,
+        "grouped_gemm_lowering": GROUPED_GEMM_LOWERING,
+        "implementation": IMPLEMENTATION,
+        "arch": ARCH,
+        "library_cache": status,
+        "library_sha256": sha,
+    }
+
+
 def _requested_ops(request: KernelRequest) -> tuple[str, ...]:
     # the order of registry.py:230-237
     ops = ["rmsnorm", "attention", "swiglu"]

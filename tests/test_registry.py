@@ -194,3 +194,19 @@ def test_torch_composition_matches_a_dense_evaluation_on_cpu():
     want = want + (torch.nn.functional.silu(x @ shared[0]) * (x @ shared[1])) @ shared[2]
     assert ids.dtype == torch.int32 and (ids.long() == torch.topk(scores, K).indices).all()
     torch.testing.assert_close(y, want, rtol=1e-5, atol=1e-5)
+
+
+def test_expert_execution_payload_names_the_lowering_and_the_library(tmp_path):
+    """The counterpart of the reference's `expert_execution` / `grouped_gemm_lowering` fields
+    (execution.py:136-138), which enter its resume fingerprint (resume.py:87-97, 115)."""
+    missing = registry.expert_execution_payload(tmp_path)
+    assert missing["expert_execution"] == "expert_major_jtmoe_grouped_gemm"
+    assert missing["grouped_gemm_lowering"] == "hip_gfx950_lds_dma_mfma"
+    assert missing["library_cache"] == "missing" and missing["library_sha256"] is None
+    built = registry.expert_execution_payload()
+    status, _ = registry.library_cache_status()
+    assert built["library_cache"] == status
+    if status == "cached":
+        assert isinstance(built["library_sha256"], str) and len(built["library_sha256"]) == 64
+    # the payload is plain JSON and stable between calls
+    assert json.dumps(built, sort_keys=True) == json.dumps(registry.expert_execution_payload(), sort_keys=True)
