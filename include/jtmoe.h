@@ -176,6 +176,23 @@ int jtmoe_sequence_balance_loss(const int32_t* expert_ids, const float* scores,
                                 float* loss, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * SMEBU balancing update: the consumer of expert_counts.  Replaces apply_moe_balance_update
+ * (steps/moe_balance.py:97-162) and the bias write of _update_expert_biases (:174-184) for L MoE
+ * layers of E experts, on device buffers (hand the layer calls rows of one [L,E] counts buffer as
+ * their expert_counts output and nothing passes through the host):
+ *   mean = sum(counts)/E; violation = (mean - counts)/max(mean, 1e-6);
+ *   delta = load_lr * tanh(clamp * violation); delta -= mean(delta);
+ *   momentum = momentum_factor * momentum + (1 - momentum_factor) * delta;  expert_bias += momentum.
+ *   router_counts [L,E] f32; momentum, expert_bias [L,E] f32, updated in place;
+ *   metrics6 = {max_vio (max over layers), load_min, load_max, load_entropy (mean over layers),
+ *               bias_norm, momentum_norm}  (MoeBalanceMetrics, :32-41).
+ *   load_lr, momentum_factor, clamp > 0 (MoeBalanceSpec, specs/model.py:18-36).
+ */
+int jtmoe_smebu_update(const float* router_counts, float* momentum, float* expert_bias,
+                       int64_t L, int64_t E, float load_lr, float momentum_factor, float clamp,
+                       float* metrics6, void* stream);
+
+/*
  * The whole layer.  Replaces SparseMoE.__call__ / forward_with_output
  * (moe.py:411-446): router -> dispatch -> grouped SwiGLU -> (shared experts) ->
  * combine, enqueued back to back on `stream`.

@@ -14,6 +14,7 @@ in NumPy, the algorithm of the reference layer
 * ``router_stats``      <- ``_router_stats``                     moe.py:794-825
 * ``sequence_balance_loss`` <- ``_sequence_balance_loss``        moe.py:828-840
 * ``moe_forward``       <- ``SparseMoE.forward_with_output``     moe.py:418-446
+* ``smebu_update``      <- ``apply_moe_balance_update``          steps/moe_balance.py:97-162, 174-184
 * ``rmsnorm`` / ``ffn_block_forward`` <- the block around the layer  blocks.py:224-230, norm.py:12-31
 
 The arithmetic the reference delegates to jax 0.10.0 / jaxlib 0.10.0 (pinned
@@ -50,6 +51,12 @@ Parity status of each function (what pins it is exercised in
 * shared_swiglu: pinned by test_model.py:873-884 (zeroed routed experts).
 * router_stats / sequence_balance_loss: pinned by test_model.py:242-252 and
   :905-908 and closed forms.
+* smebu_update: pinned by a hand-computed two-expert case in float64, the reference's two
+  train-step properties (tests/jaxtitan/test_train_step.py:352-388: from a zero state the updated
+  bias equals the momentum and is non-zero; :391-418: doubling every count leaves the momentum
+  unchanged), and invariants (balanced counts give a pure momentum decay; the centred deltas sum to
+  zero; overloaded experts move down, underloaded ones up; the metrics equal the router
+  statistics of each layer).
 * rmsnorm: pinned by the reference's known-answer test (tests/jaxtitan/test_kernels.py:192-204),
   a float64 closed form and the scale-invariance property rmsnorm(c x) = rmsnorm(x) at eps = 0.
   Which of two equally valid fp32 multiplication orders flax uses: PARITY UNPINNED at the
@@ -423,6 +430,77 @@ def sequence_balance_loss(expert_ids: np.ndarray, scores: np.ndarray, top_k: int
     normalized = scores / np.maximum(scores.sum(axis=-1, keepdims=True, dtype=np.float32), F32(1e-20))
     p_i = normalized.mean(axis=1, dtype=np.float32)
     return np.float32(np.sum(f_i * p_i, dtype=np.float32) / F32(batch))
+
+
+# --------------------------------------------------------------------------
+# SMEBU balancing update, the consumer of expert_counts  (steps/moe_balance.py:97-162)
+# --------------------------------------------------------------------------
+@dataclass
+class SmebuResult:
+    momentum: np.ndarray  # [L,E] float32
+    expert_bias: np.ndarray  # [L,E] float32
+    max_vio: np.float32  # max over layers
+    load_min: np.float32  # min over layers
+    load_max: np.float32  # max over layers
+    load_entropy: np.float32  # mean over layers
+    bias_norm: np.float32  # sqrt of the sum of squares of every updated bias
+    momentum_norm: np.float32
+
+
+def smebu_update(
+    router_counts: np.ndarray,
+    momentum: np.ndarray,
+    expert_bias: np.ndarray,
+    load_lr: float,
+    momentum_factor: float,
+    clamp: float,
+) -> SmebuResult:
+    """One non-gradient balancing step for L layers of E experts, all in float32.
+
+    Per layer (steps/moe_balance.py:123-146): mean = sum(counts)/E; violation = (mean - counts) /
+    max(mean, 1e-6); delta = load_lr * tanh(clamp * violation); delta -= mean(delta);
+    momentum' = f * momentum + (1 - f) * delta; bias' = f32(bias) + momentum' (:180);
+    metrics as in :139-161.
+    """
+    counts = np.asarray(router_counts, dtype=np.float32)
+    momentum = np.asarray(momentum, dtype=np.float32)
+    bias = np.asarray(expert_bias, dtype=np.float32)
+    if counts.ndim != 2 or counts.shape != momentum.shape or counts.shape != bias.shape:
+        raise ValueError("router count shape must match MoE balance state")
+    layers, num_experts = counts.shape
+    lr, factor, cl = F32(load_lr), F32(momentum_factor), F32(clamp)
+    next_momentum = np.empty_like(momentum)
+    next_bias = np.empty_like(bias)
+    max_vios, mins, maxes, entropies = [], [], [], []
+    bias_sq = F32(0.0)
+    momentum_sq = F32(0.0)
+    for layer in range(layers):
+        c = counts[layer]
+        count_sum = np.float32(c.sum(dtype=np.float32))
+        mean = np.float32(count_sum / F32(num_experts))
+        violation = (mean - c) / np.maximum(mean, F32(1e-6))
+        delta = lr * np.tanh(cl * violation)
+        delta = delta - np.float32(delta.mean(dtype=np.float32))
+        m = factor * momentum[layer] + (F32(1.0) - factor) * delta
+        next_momentum[layer] = m
+        next_bias[layer] = bias[layer] + m
+        st = stats_from_counts(c, np.zeros_like(c))
+        max_vios.append(st.max_vio)
+        mins.append(st.load_min)
+        maxes.append(st.load_max)
+        entropies.append(st.load_entropy)
+        momentum_sq = np.float32(momentum_sq + np.sum(np.square(m), dtype=np.float32))
+        bias_sq = np.float32(bias_sq + np.sum(np.square(next_bias[layer]), dtype=np.float32))
+    return SmebuResult(
+        next_momentum,
+        next_bias,
+        np.float32(max(max_vios)),
+        np.float32(min(mins)),
+        np.float32(max(maxes)),
+        np.float32(np.mean(np.asarray(entropies, dtype=np.float32), dtype=np.float32)),
+        np.float32(np.sqrt(bias_sq)),
+        np.float32(np.sqrt(momentum_sq)),
+    )
 
 
 # --------------------------------------------------------------------------

@@ -20,6 +20,7 @@ c_ptr = ctypes.c_void_p
 c_size = ctypes.c_size_t
 c_int = ctypes.c_int
 c_dbl = ctypes.c_double
+c_float = ctypes.c_float
 
 # symbol -> (restype, argtypes); exactly the entry points of include/jtmoe.h
 PROTOTYPES: dict[str, tuple] = {
@@ -52,6 +53,7 @@ PROTOTYPES: dict[str, tuple] = {
     "jtmoe_shared_swiglu": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr]),
     "jtmoe_combine": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr]),
     "jtmoe_router_stats": (c_int, [c_ptr, c_i64, c_ptr, c_ptr]),
+    "jtmoe_smebu_update": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_float, c_float, c_float, c_ptr, c_ptr]),
     "jtmoe_balance_workspace_bytes": (c_size, [c_i64, c_i64]),
     "jtmoe_sequence_balance_loss": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
     "jtmoe_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),

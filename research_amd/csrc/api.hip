@@ -154,6 +154,92 @@ __global__ __launch_bounds__(256) void router_stats_kernel(const float* __restri
   }
 }
 
+// ---- SMEBU balancing update (reference steps/moe_balance.py:123-161, 174-184) ----------------
+// One workgroup walks the layers in order.  Per layer: mean = sum(counts) / E;
+// violation = (mean - counts) / max(mean, 1e-6); delta = load_lr * tanh(clamp * violation), centred on
+// its mean; momentum' = f * momentum + (1 - f) * delta; bias' = bias + momentum'.
+// metrics = {max over layers of max_vio, min of load_min, max of load_max, mean of the load entropy,
+//            sqrt(sum bias'^2), sqrt(sum momentum'^2)}.  All sums are taken in a fixed order.
+__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
+  const int tid = threadIdx.x;
+  __syncthreads();  // the previous use of the scratch is over
+  scratch[tid] = v;
+  __syncthreads();
+  for (int d = 128; d >= 1; d >>= 1) {
+    if (tid < d) scratch[tid] += scratch[tid + d];
+    __syncthreads();
+  }
+  return scratch[0];
+}
+
+__global__ __launch_bounds__(256) void smebu_update_kernel(const float* __restrict__ counts, float* __restrict__ momentum,
+                                                           float* __restrict__ bias, int L, int E, float load_lr,
+                                                           float factor, float clamp, float* __restrict__ metrics) {
+  __shared__ float s_sum[256], s_min[256], s_max[256];
+  const int tid = threadIdx.x;
+  float all_vio = -3.402823466e38f, all_min = 3.402823466e38f, all_max = -3.402823466e38f;
+  float entropy_sum = 0.0f, bias_sq = 0.0f, momentum_sq = 0.0f;
+  for (int l = 0; l < L; ++l) {
+    const float* c = counts + (size_t)l * E;
+    float* m = momentum + (size_t)l * E;
+    float* b = bias + (size_t)l * E;
+    float sum = 0.0f, mn = 3.402823466e38f, mx = -3.402823466e38f;
+    for (int e = tid; e < E; e += 256) {
+      const float v = c[e];
+      sum += v;
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+    __syncthreads();
+    s_min[tid] = mn;
+    s_max[tid] = mx;
+    const float total = block_sum_256(sum, s_sum);  // its barriers also order the two arrays above
+    for (int d = 128; d >= 1; d >>= 1) {
+      if (tid < d) {
+        s_min[tid] = fminf(s_min[tid], s_min[tid + d]);
+        s_max[tid] = fmaxf(s_max[tid], s_max[tid + d]);
+      }
+      __syncthreads();
+    }
+    const float lmin = s_min[0], lmax = s_max[0];
+    const float mean = total / (float)E;
+    const float denom = fmaxf(mean, 1e-6f);
+    float dsum = 0.0f;
+    for (int e = tid; e < E; e += 256) dsum += load_lr * tanhf(clamp * ((mean - c[e]) / denom));
+    const float dmean = block_sum_256(dsum, s_sum) / (float)E;
+    float ent = 0.0f, bsq = 0.0f, msq = 0.0f;
+    const float pden = fmaxf(total, 1e-6f);
+    for (int e = tid; e < E; e += 256) {
+      const float delta = load_lr * tanhf(clamp * ((mean - c[e]) / denom)) - dmean;
+      const float next_m = factor * m[e] + (1.0f - factor) * delta;
+      const float next_b = b[e] + next_m;
+      m[e] = next_m;
+      b[e] = next_b;
+      msq += next_m * next_m;
+      bsq += next_b * next_b;
+      const float p = c[e] / pden;
+      if (p > 0.0f) ent += p * logf(p);
+    }
+    ent = block_sum_256(ent, s_sum);
+    bsq = block_sum_256(bsq, s_sum);
+    msq = block_sum_256(msq, s_sum);
+    all_vio = fmaxf(all_vio, (lmax - mean) / denom);
+    all_min = fminf(all_min, lmin);
+    all_max = fmaxf(all_max, lmax);
+    entropy_sum += -ent;
+    bias_sq += bsq;
+    momentum_sq += msq;
+  }
+  if (tid == 0) {
+    metrics[0] = all_vio;
+    metrics[1] = all_min;
+    metrics[2] = all_max;
+    metrics[3] = entropy_sum / (float)L;
+    metrics[4] = sqrtf(bias_sq);
+    metrics[5] = sqrtf(momentum_sq);
+  }
+}
+
 struct Carve {
   unsigned char* base;
   size_t used;
@@ -237,6 +323,20 @@ extern "C" int jtmoe_router_stats(const float* expert_counts, int64_t E, float* 
   JT_REQUIRE(expert_counts && stats6, "router_stats: null pointer argument");
   router_stats_kernel<<<1, 256, 0, as_stream(stream)>>>(expert_counts, (int)E, stats6);
   return check_launch("router_stats");
+}
+
+extern "C" int jtmoe_smebu_update(const float* router_counts, float* momentum, float* expert_bias, int64_t L,
+                                  int64_t E, float load_lr, float momentum_factor, float clamp, float* metrics6,
+                                  void* stream) {
+  clear_error();
+  JT_REQUIRE(L > 0 && L < ((int64_t)1 << 20) && E > 0 && E < ((int64_t)1 << 24), "smebu_update: L=%lld E=%lld out of range",
+             (long long)L, (long long)E);
+  JT_REQUIRE(load_lr > 0.0f && momentum_factor > 0.0f && clamp > 0.0f,
+             "smebu_update: load_lr, momentum and clamp must be positive");
+  JT_REQUIRE(router_counts && momentum && expert_bias && metrics6, "smebu_update: null pointer argument");
+  smebu_update_kernel<<<1, 256, 0, as_stream(stream)>>>(router_counts, momentum, expert_bias, (int)L, (int)E, load_lr,
+                                                       momentum_factor, clamp, metrics6);
+  return check_launch("smebu_update");
 }
 
 extern "C" size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,

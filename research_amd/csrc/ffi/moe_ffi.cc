@@ -285,6 +285,35 @@ ffi::Error FfnBlockForward(hipStream_t stream, ffi::AnyBuffer x, ffi::Buffer<ffi
   return status_to_error(rc);
 }
 
+// SMEBU balancing update (steps/moe_balance.py:97-162).  The C entry point works in place; XLA hands
+// over separate result buffers unless the caller aliases operands 1 and 2 to results 0 and 1
+// (input_output_aliases), so the state is copied across first when the pointers differ.
+ffi::Error MoeSmebuUpdate(hipStream_t stream, ffi::Buffer<ffi::DataType::F32> router_counts,
+                          ffi::Buffer<ffi::DataType::F32> momentum, ffi::Buffer<ffi::DataType::F32> expert_bias,
+                          ffi::Result<ffi::Buffer<ffi::DataType::F32>> next_momentum,
+                          ffi::Result<ffi::Buffer<ffi::DataType::F32>> next_bias,
+                          ffi::Result<ffi::Buffer<ffi::DataType::F32>> metrics, double load_lr, double momentum_factor,
+                          double clamp) {
+  const auto cd = router_counts.dimensions();
+  if (cd.size() != 2) return ffi::Error::InvalidArgument("router counts must have shape [layers, experts]");
+  const size_t n = router_counts.element_count();
+  if (momentum.element_count() != n || expert_bias.element_count() != n || next_momentum->element_count() != n ||
+      next_bias->element_count() != n)
+    return ffi::Error::InvalidArgument("router count shape must match MoE balance state");
+  if (metrics->element_count() != 6) return ffi::Error::InvalidArgument("metrics must have shape [6]");
+  if (next_momentum->typed_data() != momentum.typed_data() &&
+      hipMemcpyAsync(next_momentum->typed_data(), momentum.typed_data(), n * sizeof(float), hipMemcpyDeviceToDevice,
+                     stream) != hipSuccess)
+    return ffi::Error::Internal("smebu update: copy of the momentum failed");
+  if (next_bias->typed_data() != expert_bias.typed_data() &&
+      hipMemcpyAsync(next_bias->typed_data(), expert_bias.typed_data(), n * sizeof(float), hipMemcpyDeviceToDevice,
+                     stream) != hipSuccess)
+    return ffi::Error::Internal("smebu update: copy of the expert bias failed");
+  return status_to_error(jtmoe_smebu_update(router_counts.typed_data(), next_momentum->typed_data(),
+                                            next_bias->typed_data(), cd[0], cd[1], (float)load_lr,
+                                            (float)momentum_factor, (float)clamp, metrics->typed_data(), stream));
+}
+
 }  // namespace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanMoeForward, MoeForward,
@@ -406,6 +435,15 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanFfnBlockForward, FfnBlockForward,
                                   .Attr<int64_t>("top_k")
                                   .Attr<double>("route_scale")
                                   .Attr<double>("eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(JaxtitanMoeSmebuUpdate, MoeSmebuUpdate,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  JT_F32 JT_F32 JT_F32    // router counts, momentum, expert bias
+                                  JT_RF32 JT_RF32 JT_RF32  // next momentum, next bias, metrics
+                                  .Attr<double>("load_lr")
+                                  .Attr<double>("momentum_factor")
+                                  .Attr<double>("clamp"));
 
 #undef JT_ANY
 #undef JT_F32

@@ -28,6 +28,7 @@ TARGETS = {
     "jaxtitan_moe_backward": "JaxtitanMoeBackward",
     "jaxtitan_rmsnorm": "JaxtitanRmsnorm",
     "jaxtitan_ffn_block_forward": "JaxtitanFfnBlockForward",
+    "jaxtitan_moe_smebu_update": "JaxtitanMoeSmebuUpdate",
 }
 
 _REGISTERED: set[str] = set()
@@ -101,6 +102,28 @@ def moe_forward(x: Any, router_kernel: Any, expert_bias: Any, gate: Any, up: Any
     out = call(x, router_kernel, expert_bias, gate, up, down, *shared, top_k=int(top_k),
                route_scale=float(route_scale))
     return out[:6]
+
+
+def smebu_update(router_counts: Any, momentum: Any, expert_bias: Any, *, load_lr: float, momentum_factor: float,
+                 clamp: float, cache_root: str | Path | None = None):
+    """The per-layer arithmetic of apply_moe_balance_update (steps/moe_balance.py:123-161) on stacked
+    [layers, experts] f32 arrays: returns (next_momentum, next_expert_bias, metrics[6]).  The state
+    operands are aliased to the results, so under jit with donated state nothing is copied."""
+    jax = _jax()
+    import jax.numpy as jnp  # noqa: PLC0415
+
+    register_moe(cache_root)
+    if router_counts.ndim != 2 or router_counts.shape != momentum.shape or router_counts.shape != expert_bias.shape:
+        raise ContractError(f"router count shape must match MoE balance state, got {router_counts.shape}")
+    sds = jax.ShapeDtypeStruct
+    call = jax.ffi.ffi_call(
+        "jaxtitan_moe_smebu_update",
+        (sds(momentum.shape, jnp.float32), sds(expert_bias.shape, jnp.float32), sds((6,), jnp.float32)),
+        input_output_aliases={1: 0, 2: 1},
+        vmap_method="sequential",
+    )
+    return call(router_counts.astype(jnp.float32), momentum.astype(jnp.float32), expert_bias.astype(jnp.float32),
+                load_lr=float(load_lr), momentum_factor=float(momentum_factor), clamp=float(clamp))
 
 
 def moe_layer(x: Any, router_kernel: Any, expert_bias: Any, gate: Any, up: Any, down: Any, *, top_k: int,

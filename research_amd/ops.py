@@ -385,6 +385,27 @@ def router_stats(expert_counts: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def smebu_update(router_counts: torch.Tensor, momentum: torch.Tensor, expert_bias: torch.Tensor, *, load_lr: float,
+                 momentum_factor: float, clamp: float) -> torch.Tensor:
+    """One SMEBU step on device: router_counts [L,E] f32 -> momentum, expert_bias [L,E] f32 updated in place.
+
+    Returns [6] f32: max_vio, load_min, load_max, load_entropy, bias_norm, momentum_norm
+    (steps/moe_balance.py:97-162).
+    """
+    _check(router_counts, "router_counts", torch.float32)
+    if router_counts.dim() != 2 or router_counts.numel() == 0:
+        raise ContractError(f"router_counts must have shape [layers, experts], got {list(router_counts.shape)}")
+    layers, experts = router_counts.shape
+    _check(momentum, "momentum", torch.float32, (layers, experts))
+    _check(expert_bias, "expert_bias", torch.float32, (layers, experts))
+    out = torch.empty((6,), dtype=torch.float32, device=router_counts.device)
+    status = _lib().jtmoe_smebu_update(_ptr(router_counts), _ptr(momentum), _ptr(expert_bias), layers, experts,
+                                       float(load_lr), float(momentum_factor), float(clamp), _ptr(out),
+                                       _stream(out.device))
+    _raise(status, "jtmoe_smebu_update")
+    return out
+
+
 def sequence_balance_loss(expert_ids: torch.Tensor, scores: torch.Tensor, *, top_k: int) -> torch.Tensor:
     """expert_ids [B,S,K] int32, scores [B,S,E] f32 -> scalar f32 tensor."""
     if not isinstance(scores, torch.Tensor) or scores.dim() != 3:
@@ -446,8 +467,12 @@ def moe_forward(
     shared: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
     workspace: torch.Tensor | None = None,
     stage_ms: list | None = None,
+    expert_counts_out: torch.Tensor | None = None,
 ) -> LayerResult:
     """The whole layer on x [T,H] through the single C entry point jtmoe_moe_forward.
+
+    ``expert_counts_out`` ([experts] f32, contiguous — e.g. one row of the [layers, experts] buffer
+    the balancing update reads) receives the expert counts instead of a fresh tensor.
 
     With ``stage_ms`` (a list) the measuring variant jtmoe_moe_forward_timed is
     used instead: it synchronises the stream and the list receives the elapsed
@@ -489,7 +514,11 @@ def moe_forward(
     expert_ids = torch.empty((tokens, top_k), dtype=i32, device=dev)
     weights = torch.empty((tokens, top_k), dtype=x.dtype, device=dev)
     scores = torch.empty((tokens, experts), dtype=f32, device=dev)
-    expert_counts = torch.empty((experts,), dtype=f32, device=dev)
+    if expert_counts_out is None:
+        expert_counts = torch.empty((experts,), dtype=f32, device=dev)
+    else:
+        _check(expert_counts_out, "expert_counts_out", f32, (experts,))
+        expert_counts = expert_counts_out
     importance = torch.empty((experts,), dtype=f32, device=dev)
     group_sizes = torch.empty((experts,), dtype=i32, device=dev)
     offsets = torch.empty((experts,), dtype=i32, device=dev)

@@ -74,7 +74,7 @@ def test_jax_ffi_stub_fails_loudly_without_jax():
     assert set(jax_ffi.TARGETS.values()) == {
         "JaxtitanMoeForward", "JaxtitanMoeRouter", "JaxtitanMoeDispatch", "JaxtitanMoeGroupedSwiglu",
         "JaxtitanMoeCombine", "JaxtitanMoeForwardTrain", "JaxtitanMoeBackward", "JaxtitanRmsnorm",
-        "JaxtitanFfnBlockForward"}
+        "JaxtitanFfnBlockForward", "JaxtitanMoeSmebuUpdate"}
     with pytest.raises(ContractError, match="jax is not installed"):
         jax_ffi.moe_layer(None, None, None, None, None, None, top_k=1)
 
@@ -96,3 +96,32 @@ def test_training_and_block_operators_refuse_cpu_tensors_and_bad_shapes():
         ops.ffn_block_forward(x, torch.ones(8), torch.ones(8), 1e-6, torch.zeros((8, 2)), None, gate, up, down, 1)
     with pytest.raises(ContractError, match="GPU"):
         grad.moe_forward_train(x, torch.zeros((8, 2)), None, gate, up, down, 1)
+
+
+def test_balance_spec_and_state_contract():
+    """The policy checks of the reference's MoeBalanceSpec (specs/model.py:25-42) and of
+    initialize_moe_balance_state (steps/moe_balance.py:44-63), which need no GPU."""
+    import torch
+
+    from research_amd import balance as B
+
+    assert B.MoeBalanceSpec().name == "none" and B.MoeBalanceSpec(name="smebu").load_lr == 5e-4
+    with pytest.raises(ContractError, match="balance.name must be one of"):
+        B.MoeBalanceSpec(name="aux_free")
+    for field in ("load_lr", "momentum", "clamp"):
+        with pytest.raises(ContractError, match=f"balance.{field} must be positive"):
+            B.MoeBalanceSpec(name="smebu", **{field: 0.0})
+        with pytest.raises(ContractError, match=f"balance.{field} must be positive"):
+            B.MoeBalanceSpec(name="smebu", **{field: True})
+    with pytest.raises(ContractError, match="sequence_aux_loss_weight must be non-negative"):
+        B.MoeBalanceSpec(name="smebu", sequence_aux_loss_weight=-1.0)
+    bias = torch.zeros((3, 8))
+    assert B.initialize_moe_balance_state(bias, None) is None
+    assert B.initialize_moe_balance_state(bias, B.MoeBalanceSpec()) is None
+    state = B.initialize_moe_balance_state(bias, B.MoeBalanceSpec(name="smebu", momentum=0.25))
+    assert state.num_layers == 3 and state.momentum_factor == 0.25 and state.momentum.shape == (3, 8)
+    assert state.momentum.dtype == torch.float32 and not bool(state.momentum.any())
+    with pytest.raises(ContractError, match="requires at least one MoE expert_bias parameter"):
+        B.initialize_moe_balance_state(torch.zeros((0, 8)), B.MoeBalanceSpec(name="smebu"))
+    assert B.zero_router_counts(None).shape == (0, 0)
+    assert B.zero_router_counts(state).shape == (3, 8)
