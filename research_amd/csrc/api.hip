@@ -155,82 +155,93 @@ __global__ __launch_bounds__(256) void router_stats_kernel(const float* __restri
 }
 
 // ---- SMEBU balancing update (reference steps/moe_balance.py:123-161, 174-184) ----------------
-// One workgroup walks the layers in order.  Per layer: mean = sum(counts) / E;
+// One workgroup of 16 waves; a wave owns a layer at a time and reduces over its experts with
+// shuffles (no barriers inside a layer).  Per layer: mean = sum(counts) / E;
 // violation = (mean - counts) / max(mean, 1e-6); delta = load_lr * tanh(clamp * violation), centred on
 // its mean; momentum' = f * momentum + (1 - f) * delta; bias' = bias + momentum'.
 // metrics = {max over layers of max_vio, min of load_min, max of load_max, mean of the load entropy,
-//            sqrt(sum bias'^2), sqrt(sum momentum'^2)}.  All sums are taken in a fixed order.
-__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
-  const int tid = threadIdx.x;
-  __syncthreads();  // the previous use of the scratch is over
-  scratch[tid] = v;
-  __syncthreads();
-  for (int d = 128; d >= 1; d >>= 1) {
-    if (tid < d) scratch[tid] += scratch[tid + d];
-    __syncthreads();
-  }
-  return scratch[0];
+//            sqrt(sum bias'^2), sqrt(sum momentum'^2)}.  Every sum has a fixed order: a lane adds its
+// experts in ascending order, the wave combines lanes in a butterfly, thread 0 adds layers in order.
+constexpr int kSmebuWaves = 16;
+
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
+  return v;
 }
 
-__global__ __launch_bounds__(256) void smebu_update_kernel(const float* __restrict__ counts, float* __restrict__ momentum,
-                                                           float* __restrict__ bias, int L, int E, float load_lr,
-                                                           float factor, float clamp, float* __restrict__ metrics) {
-  __shared__ float s_sum[256], s_min[256], s_max[256];
-  const int tid = threadIdx.x;
+__global__ __launch_bounds__(kSmebuWaves * 64) void smebu_update_kernel(
+    const float* __restrict__ counts, float* __restrict__ momentum, float* __restrict__ bias, int L, int E,
+    float load_lr, float factor, float clamp, float* __restrict__ metrics) {
+  __shared__ float s_vio[kSmebuWaves], s_min[kSmebuWaves], s_max[kSmebuWaves], s_ent[kSmebuWaves],
+      s_bsq[kSmebuWaves], s_msq[kSmebuWaves];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float all_vio = -3.402823466e38f, all_min = 3.402823466e38f, all_max = -3.402823466e38f;
-  float entropy_sum = 0.0f, bias_sq = 0.0f, momentum_sq = 0.0f;
-  for (int l = 0; l < L; ++l) {
-    const float* c = counts + (size_t)l * E;
-    float* m = momentum + (size_t)l * E;
-    float* b = bias + (size_t)l * E;
-    float sum = 0.0f, mn = 3.402823466e38f, mx = -3.402823466e38f;
-    for (int e = tid; e < E; e += 256) {
-      const float v = c[e];
-      sum += v;
-      mn = fminf(mn, v);
-      mx = fmaxf(mx, v);
+  float entropy_sum = 0.0f, bias_sq = 0.0f, momentum_sq = 0.0f;  // kept by thread 0
+  for (int l0 = 0; l0 < L; l0 += kSmebuWaves) {
+    const int l = l0 + wave;
+    if (l < L) {
+      const float* c = counts + (size_t)l * E;
+      float* m = momentum + (size_t)l * E;
+      float* b = bias + (size_t)l * E;
+      float sum = 0.0f, mn = 3.402823466e38f, mx = -3.402823466e38f;
+      for (int e = lane; e < E; e += 64) {
+        const float v = c[e];
+        sum += v;
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
+      }
+      const float total = wave_sum_f32(sum);
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) {
+        mn = fminf(mn, __shfl_xor(mn, d));
+        mx = fmaxf(mx, __shfl_xor(mx, d));
+      }
+      const float mean = total / (float)E;
+      const float denom = fmaxf(mean, 1e-6f);
+      float dsum = 0.0f;
+      for (int e = lane; e < E; e += 64) dsum += load_lr * tanhf(clamp * ((mean - c[e]) / denom));
+      const float dmean = wave_sum_f32(dsum) / (float)E;
+      float ent = 0.0f, bsq = 0.0f, msq = 0.0f;
+      const float pden = fmaxf(total, 1e-6f);
+      for (int e = lane; e < E; e += 64) {
+        const float delta = load_lr * tanhf(clamp * ((mean - c[e]) / denom)) - dmean;
+        const float next_m = factor * m[e] + (1.0f - factor) * delta;
+        const float next_b = b[e] + next_m;
+        m[e] = next_m;
+        b[e] = next_b;
+        msq += next_m * next_m;
+        bsq += next_b * next_b;
+        const float p = c[e] / pden;
+        if (p > 0.0f) ent += p * logf(p);
+      }
+      ent = wave_sum_f32(ent);
+      bsq = wave_sum_f32(bsq);
+      msq = wave_sum_f32(msq);
+      if (lane == 0) {
+        s_vio[wave] = (mx - mean) / denom;
+        s_min[wave] = mn;
+        s_max[wave] = mx;
+        s_ent[wave] = -ent;
+        s_bsq[wave] = bsq;
+        s_msq[wave] = msq;
+      }
     }
     __syncthreads();
-    s_min[tid] = mn;
-    s_max[tid] = mx;
-    const float total = block_sum_256(sum, s_sum);  // its barriers also order the two arrays above
-    for (int d = 128; d >= 1; d >>= 1) {
-      if (tid < d) {
-        s_min[tid] = fminf(s_min[tid], s_min[tid + d]);
-        s_max[tid] = fmaxf(s_max[tid], s_max[tid + d]);
+    if (threadIdx.x == 0) {
+      const int n = min(kSmebuWaves, L - l0);
+      for (int w = 0; w < n; ++w) {
+        all_vio = fmaxf(all_vio, s_vio[w]);
+        all_min = fminf(all_min, s_min[w]);
+        all_max = fmaxf(all_max, s_max[w]);
+        entropy_sum += s_ent[w];
+        bias_sq += s_bsq[w];
+        momentum_sq += s_msq[w];
       }
-      __syncthreads();
     }
-    const float lmin = s_min[0], lmax = s_max[0];
-    const float mean = total / (float)E;
-    const float denom = fmaxf(mean, 1e-6f);
-    float dsum = 0.0f;
-    for (int e = tid; e < E; e += 256) dsum += load_lr * tanhf(clamp * ((mean - c[e]) / denom));
-    const float dmean = block_sum_256(dsum, s_sum) / (float)E;
-    float ent = 0.0f, bsq = 0.0f, msq = 0.0f;
-    const float pden = fmaxf(total, 1e-6f);
-    for (int e = tid; e < E; e += 256) {
-      const float delta = load_lr * tanhf(clamp * ((mean - c[e]) / denom)) - dmean;
-      const float next_m = factor * m[e] + (1.0f - factor) * delta;
-      const float next_b = b[e] + next_m;
-      m[e] = next_m;
-      b[e] = next_b;
-      msq += next_m * next_m;
-      bsq += next_b * next_b;
-      const float p = c[e] / pden;
-      if (p > 0.0f) ent += p * logf(p);
-    }
-    ent = block_sum_256(ent, s_sum);
-    bsq = block_sum_256(bsq, s_sum);
-    msq = block_sum_256(msq, s_sum);
-    all_vio = fmaxf(all_vio, (lmax - mean) / denom);
-    all_min = fminf(all_min, lmin);
-    all_max = fmaxf(all_max, lmax);
-    entropy_sum += -ent;
-    bias_sq += bsq;
-    momentum_sq += msq;
+    __syncthreads();
   }
-  if (tid == 0) {
+  if (threadIdx.x == 0) {
     metrics[0] = all_vio;
     metrics[1] = all_min;
     metrics[2] = all_max;
@@ -334,7 +345,7 @@ extern "C" int jtmoe_smebu_update(const float* router_counts, float* momentum, f
   JT_REQUIRE(load_lr > 0.0f && momentum_factor > 0.0f && clamp > 0.0f,
              "smebu_update: load_lr, momentum and clamp must be positive");
   JT_REQUIRE(router_counts && momentum && expert_bias && metrics6, "smebu_update: null pointer argument");
-  smebu_update_kernel<<<1, 256, 0, as_stream(stream)>>>(router_counts, momentum, expert_bias, (int)L, (int)E, load_lr,
+  smebu_update_kernel<<<1, kSmebuWaves * 64, 0, as_stream(stream)>>>(router_counts, momentum, expert_bias, (int)L, (int)E, load_lr,
                                                        momentum_factor, clamp, metrics6);
   return check_launch("smebu_update");
 }
