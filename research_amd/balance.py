@@ -100,6 +100,25 @@ def zero_router_counts(balance: MoeBalanceState | None, device: torch.device | s
     return torch.zeros_like(balance.momentum)
 
 
+def _stack_stats(router_stats: tuple[Any, ...], balance: MoeBalanceState | None, field: str) -> torch.Tensor:
+    if not router_stats:
+        return torch.zeros((0, 0), dtype=torch.float32)
+    if balance is not None and len(router_stats) != balance.num_layers:
+        raise ContractError(f"MoE balance expected {balance.num_layers} router stat entries, got {len(router_stats)}")
+    return torch.stack([getattr(stats, field).to(torch.float32) for stats in router_stats])
+
+
+def router_counts_from_stats(router_stats: tuple[Any, ...], balance: MoeBalanceState | None) -> torch.Tensor:
+    """Layer-major expert counts from the layers' RouterStats (moe_balance.py:73-83): the copying
+    alternative to handing the layers rows of `zero_router_counts`."""
+    return _stack_stats(router_stats, balance, "expert_counts")
+
+
+def router_importance_from_stats(router_stats: tuple[Any, ...], balance: MoeBalanceState | None) -> torch.Tensor:
+    """Layer-major selected-router-weight sums from the layers' RouterStats (moe_balance.py:86-94)."""
+    return _stack_stats(router_stats, balance, "importance")
+
+
 def apply_moe_balance_update(
     expert_bias: torch.Tensor,
     balance: MoeBalanceState | None,

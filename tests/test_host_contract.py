@@ -125,3 +125,13 @@ def test_balance_spec_and_state_contract():
         B.initialize_moe_balance_state(torch.zeros((0, 8)), B.MoeBalanceSpec(name="smebu"))
     assert B.zero_router_counts(None).shape == (0, 0)
     assert B.zero_router_counts(state).shape == (3, 8)
+    # stacking the layers' statistics (moe_balance.py:73-94)
+    from types import SimpleNamespace
+
+    stats = tuple(SimpleNamespace(expert_counts=torch.full((8,), float(i)), importance=torch.full((8,), 0.5 * i))
+                  for i in range(3))
+    assert B.router_counts_from_stats(stats, state)[2].tolist() == [2.0] * 8
+    assert B.router_importance_from_stats(stats, state).shape == (3, 8)
+    assert B.router_counts_from_stats((), state).shape == (0, 0)
+    with pytest.raises(ContractError, match="MoE balance expected 3 router stat entries, got 2"):
+        B.router_counts_from_stats(stats[:2], state)
