@@ -159,7 +159,8 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
                 const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream,
                 const int32_t* row_map = nullptr, int row_div = 1, int64_t a_rows = 0, void* save0 = nullptr,
                 void* save1 = nullptr) {
-  // the 256-row configurations run as one persistent workgroup per CU, the others one tile per workgroup
+  // the 256-row configurations run as persistent workgroups (see persistent_schedule), the others one
+  // tile per workgroup
   constexpr bool kPersistent = Cfg::BM == 256 && Cfg::NSTAGE == 2 && Cfg::BK == 64;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
@@ -180,11 +181,19 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   const int64_t nt = (N + Cfg::BN - 1) / Cfg::BN;
   const int64_t tiles_grid = gemm_grid(mtiles, nt);
   if (tiles_grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
-  const int64_t grid = kPersistent && tiles_grid > persistent_grid_size() ? persistent_grid_size() : tiles_grid;
-  kernel<<<(unsigned)grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
-      static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
-      static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,
-      row_map, row_div, (int)a_rows, static_cast<uint16_t*>(save0), static_cast<uint16_t*>(save1));
+  if constexpr (kPersistent) {
+    const PersistentSchedule ps = persistent_schedule(tiles_grid, persistent_grid_size(), kTilesPerWorkgroup<Cfg>);
+    kernel<<<(unsigned)ps.grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
+        static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
+        static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,
+        row_map, row_div, (int)a_rows, static_cast<uint16_t*>(save0), static_cast<uint16_t*>(save1), ps.window,
+        ps.chunk);
+  } else {
+    kernel<<<(unsigned)tiles_grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
+        static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
+        static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,
+        row_map, row_div, (int)a_rows, static_cast<uint16_t*>(save0), static_cast<uint16_t*>(save1));
+  }
   return JTMOE_OK;
 }
 

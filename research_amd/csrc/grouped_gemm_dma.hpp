@@ -371,23 +371,31 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// The same tile computation for launches with many tiles per CU: one workgroup per CU walks a
-// sequence of tiles (the XCD's contiguous range of the logical order, with the stride of the
-// XCD's workgroups).  The tile after the current one is looked up when the current one starts, and
-// its first operand tiles are requested right after the current k loop, before the epilogue: the
-// latency of those loads, the tile look-up and the start of a new workgroup no longer stand
-// between two tiles.  At the C3 shape the down projection (22 k steps, 128 KB of results per
-// tile) goes from 0.78 to 0.735 ms, gate/up from 1.465 to 1.45 ms.
+// The same tile computation for launches with many tiles per CU: a workgroup walks a sequence of
+// tiles of its XCD's contiguous range of the logical order.  The tile after the current one is
+// looked up when the current one starts, and its first operand tiles are requested right after the
+// current k loop, before the epilogue: the latency of those loads, the tile look-up and the start
+// of a new workgroup no longer stand between two tiles.  At the C3 shape the down projection (22 k
+// steps, 128 KB of results per tile) goes from 0.78 to 0.735 ms, gate/up from 1.465 to 1.44 ms.
 // The epilogue stages results above the first stage buffer (which the next tile's loads are
 // filling), in two halves where a wave's block does not fit its share of that area.
-// Launch with a multiple of 8 workgroups (one per CU).
+// Two schedules (launch with a multiple of 8 workgroups):
+//   chunk == 0: one workgroup per CU for the whole launch; workgroup i of an XCD takes tiles
+//     i, i + n, i + 2n, ... of the range (n workgroups per XCD).
+//   chunk > 0: many workgroups of `chunk` tiles each, which the hardware starts in order as CUs
+//     become free.  With `window` workgroups resident per XCD, workgroup j takes tiles
+//     (j / window) * window * chunk + j % window + p * window, p < chunk: the resident workgroups
+//     stay within window * chunk consecutive tiles of each other, where fully persistent ones drift
+//     apart and share fewer operand panels in the L2 (gate/up at C3: 5.9 GB leave the L2 per launch
+//     with chunk 0, 4.4 GB with chunk 4, 4.1 GB with one tile per workgroup; the run time is the
+//     same for chunk 0, 2, 4 and 8).
 // ---------------------------------------------------------------------------------------------
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
     uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
     int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
-    int a_rows, uint16_t* __restrict__ save0, uint16_t* __restrict__ save1) {
+    int a_rows, uint16_t* __restrict__ save0, uint16_t* __restrict__ save1, int window, int chunk) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   constexpr int CPRA = Cfg::CPRA;
@@ -410,8 +418,13 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
   }
   const int total = real_mtiles * ntiles_n;
   const int per_xcd = (total + 7) >> 3;
-  const int xcd = (int)blockIdx.x & 7, stride = max(1, (int)gridDim.x >> 3);  // the launch uses a multiple of 8 workgroups
-  int idx = (int)blockIdx.x >> 3;
+  const int xcd = (int)blockIdx.x & 7;  // the launch uses a multiple of 8 workgroups
+  int idx = (int)blockIdx.x >> 3, stride = max(1, (int)gridDim.x >> 3), left = 0x7fffffff;
+  if (chunk > 0) {
+    idx = (idx / window) * (window * chunk) + idx % window;
+    stride = window;
+    left = chunk;
+  }
 
   struct Tile {
     int expert, row0, rows, n0;
@@ -558,7 +571,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
     // the tile after this one is looked up now, and its row offsets requested, so that nothing but the
     // issue of its first loads stands between the end of this tile's k loop and its epilogue
     idx += stride;
-    const Tile nxt = locate(idx);
+    --left;
+    const Tile nxt = locate(left > 0 ? idx : 0x3fffffff);
     int nxt_voff[Cfg::A_LOADS];
     if (nxt.rows > 0) row_offsets(nxt, nxt_voff);
 
@@ -636,10 +650,29 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
 }
 
 
+// Grid and schedule of a persistent launch over `tiles_grid` (a multiple of 8) tiles on a device with
+// `cus` CUs (a multiple of 8): see the two schedules above.
+struct PersistentSchedule {
+  int64_t grid;
+  int window, chunk;
+};
+inline PersistentSchedule persistent_schedule(int64_t tiles_grid, int cus, int tiles_per_workgroup) {
+  if (tiles_grid <= cus) return {tiles_grid, 0, 0};  // a tile per workgroup, no second tile to look up
+  if (tiles_per_workgroup <= 0) return {cus, 0, 0};
+  const int window = cus / 8;
+  const int64_t per_xcd = tiles_grid / 8, span = (int64_t)window * tiles_per_workgroup;
+  return {8 * ((per_xcd + span - 1) / span) * window, window, tiles_per_workgroup};
+}
+
 // The two configurations the library launches: 256 x 256 output tiles (gate and up share the A
 // tile: 128 + 128 columns), 64-deep k steps, two LDS stages, 8 waves, B tiles in 4 x 64 blocks
 // (whole 128-byte lines per eight lanes; about 1 % faster than 4 x 16 blocks at 131072 rows).
 using GateUpCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
+// tiles per workgroup of a persistent launch (0: one workgroup per CU walks them all).  The down
+// projection measures 0.8 % faster fully persistent (and sheds 7 % of its L2 misses with 4); gate/up
+// runs as fast either way and sheds a quarter of them.
+template <typename Cfg>
+constexpr int kTilesPerWorkgroup = Cfg::kDual ? 4 : 0;
 using DownCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128 + 32768>;  // 537 MB of results at C3: streamed out
 // Few rows per group (decode-sized batches): the layer streams every expert matrix once and
 // is bound by HBM, so the tiles are only 64 rows tall to keep the padded-row MFMA work below

@@ -122,21 +122,32 @@ static void release(Problem& p) {
 // The 256-row configurations run as the library runs them: persistent workgroups, one per CU (256
 // here), unless g_one_tile_per_workgroup asks for the plain kernel.
 static bool g_one_tile_per_workgroup = false;
+static int g_chunk = -1;  // tiles per workgroup of a persistent launch; -1: as the library chooses
 template <typename Cfg>
 static void launch(Problem& p, bool dense) {
   constexpr bool kCanPersist = Cfg::BM == 256 && Cfg::NSTAGE == 2 && Cfg::BK == 64;
   const bool persist = kCanPersist && !g_one_tile_per_workgroup;
-  auto kernel = grouped_gemm_dma_kernel<Cfg>;
-  if constexpr (kCanPersist) {
-    if (persist) kernel = grouped_gemm_dma_persistent_kernel<Cfg>;
-  }
-  CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                         (int)Cfg::SMEM_BYTES));
   const long mt = dense ? (p.rows + Cfg::BM - 1) / Cfg::BM
                         : (p.rows + Cfg::BM - 1) / Cfg::BM + (p.E < p.rows ? p.E : p.rows);
   const long nt = (p.N + Cfg::BN - 1) / Cfg::BN;
   const long tiles_grid = gemm_grid(mt, nt);
-  kernel<<<(unsigned)(persist && tiles_grid > 256 ? 256 : tiles_grid), Cfg::NT, Cfg::SMEM_BYTES>>>(
+  if constexpr (kCanPersist) {
+    if (persist) {
+      auto kernel = grouped_gemm_dma_persistent_kernel<Cfg>;
+      CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             (int)Cfg::SMEM_BYTES));
+      const PersistentSchedule ps = persistent_schedule(tiles_grid, 256, g_chunk < 0 ? kTilesPerWorkgroup<Cfg> : g_chunk);
+      kernel<<<(unsigned)ps.grid, Cfg::NT, Cfg::SMEM_BYTES>>>(
+          p.A, p.B0, Cfg::kDual ? p.B1 : nullptr, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows,
+          p.K, p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, nullptr,
+          nullptr, ps.window, ps.chunk);
+      return;
+    }
+  }
+  auto kernel = grouped_gemm_dma_kernel<Cfg>;
+  CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                         (int)Cfg::SMEM_BYTES));
+  kernel<<<(unsigned)tiles_grid, Cfg::NT, Cfg::SMEM_BYTES>>>(
       p.A, p.B0, Cfg::kDual ? p.B1 : nullptr, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows,
       p.K, p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, nullptr, nullptr);
 }
@@ -617,6 +628,15 @@ int main(int argc, char** argv) {
       g_one_tile_per_workgroup = false;
       timeit<GateUpCfg>("gate/up persistent (library)", g, 20);
       timeit<DownCfg>("down persistent (library)", d, 20);
+      for (int chunk : {0, 2, 4, 8}) {
+        g_chunk = chunk;
+        char name[64];
+        snprintf(name, sizeof name, "gate/up %d tiles per workgroup", chunk);
+        timeit<GateUpCfg>(name, g, 20);
+        snprintf(name, sizeof name, "down %d tiles per workgroup", chunk);
+        timeit<DownCfg>(name, d, 20);
+      }
+      g_chunk = -1;
     }
     release(g); release(d);
   }
