@@ -50,6 +50,15 @@ __device__ __forceinline__ SwigluGrad swiglu_grad(float z, float g, float u, flo
   return r;
 }
 
+// Packed rows that exist: the groups end at offsets[E-1] + group_sizes[E-1], which is less than the
+// number of assignments when the dispatch dropped ids outside [0, E).  Rows past that end hold
+// nothing (their entries of the permutation were never written) and are skipped.
+__device__ __forceinline__ int packed_rows_end(const int32_t* __restrict__ group_sizes,
+                                               const int32_t* __restrict__ offsets, int E, int rows) {
+  if (group_sizes == nullptr) return rows;
+  return min(rows, offsets[E - 1] + group_sizes[E - 1]);
+}
+
 // One wave per packed row.  z_dg holds Z on entry and dG on exit.  row_weight_index[j] (the
 // assignment behind packed row j) selects the route weight and the slot of d_weights; with a
 // null index (shared experts) the weight is 1 and no weight gradient is produced.
@@ -59,11 +68,14 @@ __global__ __launch_bounds__(256) void swiglu_backward_kernel(T* __restrict__ z_
                                                               const int32_t* __restrict__ row_weight_index,
                                                               const T* __restrict__ weights, int rows, int I,
                                                               T* __restrict__ dU, T* __restrict__ HW,
-                                                              T* __restrict__ d_weights) {
+                                                              T* __restrict__ d_weights,
+                                                              const int32_t* __restrict__ group_sizes,
+                                                              const int32_t* __restrict__ offsets, int E) {
   const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (j >= rows) return;
+  if (j >= packed_rows_end(group_sizes, offsets, E, rows)) return;
   const int lane = threadIdx.x & 63;
   const int a = row_weight_index ? row_weight_index[j] : 0;
+  if (a < 0 || a >= rows) return;  // not a permutation entry: nothing to read or write through it
   const float w = row_weight_index ? Elem<T>::load(weights + a) : 1.0f;
   const size_t base = (size_t)j * I;
   float dot = 0.0f;
@@ -83,11 +95,13 @@ __global__ __launch_bounds__(256) void swiglu_backward_kernel(T* __restrict__ z_
 __global__ __launch_bounds__(256) void swiglu_backward_bf16_vec_kernel(
     uint4* __restrict__ z_dg, const uint4* __restrict__ G, const uint4* __restrict__ U,
     const int32_t* __restrict__ row_weight_index, const uint16_t* __restrict__ weights, int rows, int row_vecs,
-    uint4* __restrict__ dU, uint4* __restrict__ HW, uint16_t* __restrict__ d_weights) {
+    uint4* __restrict__ dU, uint4* __restrict__ HW, uint16_t* __restrict__ d_weights,
+    const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E) {
   const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (j >= rows) return;
+  if (j >= packed_rows_end(group_sizes, offsets, E, rows)) return;
   const int lane = threadIdx.x & 63;
   const int a = row_weight_index ? row_weight_index[j] : 0;
+  if (a < 0 || a >= rows) return;
   const float w = row_weight_index ? bf16_bits_to_f32(weights[a]) : 1.0f;
   const size_t base = (size_t)j * row_vecs;
   float dot = 0.0f;
@@ -116,10 +130,15 @@ __global__ __launch_bounds__(256) void swiglu_backward_bf16_vec_kernel(
   if (row_weight_index && lane == 0) d_weights[a] = (uint16_t)f32_to_bf16_bits(dot);
 }
 
+// ones[a] = 1 (the unit weights of the combine that sums dXp), and the route-weight gradient of an
+// assignment the dispatch dropped (inverse < 0: no packed row, so no one else writes it) is zero
 template <typename T>
-__global__ __launch_bounds__(256) void fill_one_kernel(T* __restrict__ p, int n) {
+__global__ __launch_bounds__(256) void fill_one_kernel(T* __restrict__ p, int n, const int32_t* __restrict__ inverse,
+                                                       T* __restrict__ d_weights) {
   const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < n) Elem<T>::store(p + i, 1.0f);
+  if (i >= n) return;
+  Elem<T>::store(p + i, 1.0f);
+  if (inverse[i] < 0) Elem<T>::store(d_weights + i, 0.0f);
 }
 
 // out[i] = round(a[i] + b[i])
@@ -163,7 +182,8 @@ __global__ __launch_bounds__(256) void router_backward_kernel(const float* __res
 
 template <typename T>
 int run_swiglu_backward(void* z_dg, const void* G, const void* U, const int32_t* row_weight_index, const void* weights,
-                        int64_t rows, int64_t I, void* dU, void* HW, void* d_weights, hipStream_t s) {
+                        int64_t rows, int64_t I, void* dU, void* HW, void* d_weights, hipStream_t s,
+                        const int32_t* group_sizes = nullptr, const int32_t* offsets = nullptr, int64_t E = 0) {
   if (rows == 0) return JTMOE_OK;
   const unsigned grid = (unsigned)((rows + 3) / 4);
   if (Elem<T>::is_bf16 && I % 8 == 0 && aligned16(z_dg) && aligned16(G) && aligned16(U) && aligned16(dU) &&
@@ -171,13 +191,13 @@ int run_swiglu_backward(void* z_dg, const void* G, const void* U, const int32_t*
     swiglu_backward_bf16_vec_kernel<<<grid, 256, 0, s>>>(
         static_cast<uint4*>(z_dg), static_cast<const uint4*>(G), static_cast<const uint4*>(U), row_weight_index,
         static_cast<const uint16_t*>(weights), (int)rows, (int)(I / 8), static_cast<uint4*>(dU),
-        static_cast<uint4*>(HW), static_cast<uint16_t*>(d_weights));
+        static_cast<uint4*>(HW), static_cast<uint16_t*>(d_weights), group_sizes, offsets, (int)E);
   } else {
     swiglu_backward_kernel<T><<<grid, 256, 0, s>>>(static_cast<T*>(z_dg), static_cast<const T*>(G),
                                                    static_cast<const T*>(U), row_weight_index,
                                                    static_cast<const T*>(weights), (int)rows, (int)I,
                                                    static_cast<T*>(dU), static_cast<T*>(HW),
-                                                   static_cast<T*>(d_weights));
+                                                   static_cast<T*>(d_weights), group_sizes, offsets, (int)E);
   }
   return check_launch("swiglu backward");
 }
@@ -266,9 +286,9 @@ int experts_backward_core(const void* x, const void* dy, const int32_t* source_o
                       0, 1, s);
   if (rc) return rc;
   rc = dtype == JTMOE_BF16 ? run_swiglu_backward<bf16_raw>(ws.dg, gate_pre, up_pre, source_order, weights, A, I, ws.du,
-                                                           ws.hw, d_weights, s)
+                                                           ws.hw, d_weights, s, group_sizes, offsets, E)
                            : run_swiglu_backward<float>(ws.dg, gate_pre, up_pre, source_order, weights, A, I, ws.du,
-                                                        ws.hw, d_weights, s);
+                                                        ws.hw, d_weights, s, group_sizes, offsets, E);
   if (rc) return rc;
   // dWd[e] = (w Hh)^T @ dYp
   rc = launch_gemm_tn(dtype, ws.hw, ws.packed_dy, nullptr, d_down, nullptr, group_sizes, offsets, A, I, H, E, nullptr,
@@ -284,9 +304,11 @@ int experts_backward_core(const void* x, const void* dy, const int32_t* source_o
   if (A == 0) return JTMOE_OK;
   const unsigned grid = (unsigned)((A + 255) / 256);
   if (dtype == JTMOE_BF16)
-    fill_one_kernel<bf16_raw><<<grid, 256, 0, s>>>(static_cast<bf16_raw*>(ws.ones), (int)A);
+    fill_one_kernel<bf16_raw><<<grid, 256, 0, s>>>(static_cast<bf16_raw*>(ws.ones), (int)A, inverse,
+                                                   static_cast<bf16_raw*>(d_weights));
   else
-    fill_one_kernel<float><<<grid, 256, 0, s>>>(static_cast<float*>(ws.ones), (int)A);
+    fill_one_kernel<float><<<grid, 256, 0, s>>>(static_cast<float*>(ws.ones), (int)A, inverse,
+                                                static_cast<float*>(d_weights));
   return check_launch("experts backward");
 }
 

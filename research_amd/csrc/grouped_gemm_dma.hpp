@@ -39,31 +39,33 @@ __device__ __forceinline__ unsigned lds_byte_addr(const void* p) {
 }
 
 // 16 bytes per lane from a raw buffer straight into LDS at lds_base + lane*16.
-// Reads past the end of the buffer store zeros.
+// Reads past the end of the buffer store zeros.  The LDS base travels in M0; the hardware wants one
+// wait state between a scalar write of M0 and an LDS-DMA load that reads it, and the compiler's
+// hazard handling does not look inside inline assembly, so the s_nop is written out here.
 __device__ __forceinline__ void buffer_load_lds16(i32x4_t rsrc, unsigned lds_base, int voffset, int soffset) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
-               : "memory");
+               : "memory", "m0");
 }
 
 // The same with the LDS address given as a scalar base plus a compile-time offset: a kernel that
 // issues many loads per stage then keeps one scalar per stage instead of one per load.
 template <int kOffset>
 __device__ __forceinline__ void buffer_load_lds16_at(i32x4_t rsrc, unsigned lds_base, int voffset, int soffset) {
-  asm volatile("s_add_u32 m0, %0, %4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset), "n"(kOffset)
-               : "memory", "scc");
+               : "memory", "scc", "m0");
 }
 
 // The same with the non-temporal hint, for operands no other workgroup reads again (the expert
 // matrices when every group is a single tile tall).
 __device__ __forceinline__ void buffer_load_lds16_nt(i32x4_t rsrc, unsigned lds_base, int voffset, int soffset) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
                :
                : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
-               : "memory");
+               : "memory", "m0");
 }
 
 // fp32 -> bf16 by the hardware conversion (round to nearest even)

@@ -132,6 +132,50 @@ def test_expert_gradients_with_one_dominant_group(gpu, tokens, hidden, experts, 
                 assert float(np.max(np.abs(g[e] - ref[e]))) <= BF16_MAX_REL * scale, f"{tag} {name}[{e}]"
 
 
+@pytest.mark.parametrize("tokens,hidden,experts,top_k,inter,dtype",
+                         [(90, 64, 5, 2, 96, "f32"), (600, 256, 8, 4, 192, "bf16"), (3000, 128, 12, 4, 128, "bf16")])
+def test_expert_gradients_with_dropped_ids(gpu, tokens, hidden, experts, top_k, inter, dtype):
+    """Ids outside [0, E) are dropped by the dispatch (inverse = -1, fewer packed rows than assignments).
+
+    The backward pass must then stay inside the rows that exist: the gradients equal those of the
+    same problem with the dropped assignments simply absent, and the route-weight gradient of a dropped
+    assignment is exactly zero.  The buffers the tail of the plan would index are poisoned first.
+    """
+    x, gate, up, down, ids, w = random_problem(31 + tokens, tokens, hidden, experts, top_k, inter, 0.1)
+    rng = np.random.default_rng(tokens)
+    drop = rng.random(ids.shape) < 0.2
+    ids = ids.copy()
+    ids[drop] = np.where(rng.random(int(drop.sum())) < 0.5, experts + 3, -1)
+    dy = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    cast = lambda a: O.cast_compute(a, dtype)
+    want = G.experts_backward(cast(x), ids, cast(w), cast(gate), cast(up), cast(down), cast(dy))
+    assert not want.d_weights[drop].any()
+    xd, gd, ud, dd, wd, dyd = (dev(a.astype(np.float32), gpu, dtype) for a in (x, gate, up, down, w, dy))
+    plan = ops.dispatch(dev(ids.astype(np.int32), gpu), experts)
+    sizes = host(plan.group_sizes)
+    kept = int(sizes.sum())
+    assert kept == int((~drop).sum()) < tokens * top_k
+    assert np.array_equal(host(plan.inverse).reshape(ids.shape) < 0, drop)
+    # what lies past the last group is not part of the plan: make any use of it show
+    plan.source_order[kept:] = 0x3FFFFFFF
+    _, _, res = grad.grouped_swiglu_train(xd, plan.source_order, top_k, gd, ud, dd, plan.group_sizes, plan.offsets)
+    res.gate_pre[kept:] = float("nan")
+    res.up_pre[kept:] = float("nan")
+    got = grad.experts_backward(xd, dyd, plan, wd, gd, ud, dd, res)
+    again = grad.experts_backward(xd, dyd, plan, wd, gd, ud, dd, res)
+    tag = f"dropped ids {dtype} T={tokens} E={experts} K={top_k}"
+    for name in ("dx", "d_weights", "d_gate", "d_up", "d_down"):
+        g, ref = getattr(got, name), getattr(want, name).astype(np.float32)
+        assert bool(torch.isfinite(g).all()), name
+        assert torch.equal(g, getattr(again, name)), f"{name} differs between two identical calls"
+        if dtype == "bf16":
+            assert report(f"{tag} {name}", host(g), ref) <= BF16_MAX_REL
+        else:
+            scale = float(np.max(np.abs(ref))) or 1.0
+            np.testing.assert_allclose(host(g) / scale, ref / scale, rtol=1e-4, atol=2e-5, err_msg=name)
+    assert not host(got.d_weights)[drop].any()
+
+
 # the 4096-token cases take the path that splits a long one-group reduction into partial sums
 @pytest.mark.parametrize("tokens,hidden,inter,dtype", [(5, 16, 24, "f32"), (300, 1024, 704, "bf16"), (130, 72, 40, "bf16"),
                                                        (4096, 512, 704, "bf16"), (64, 1024, 704, "bf16")])
