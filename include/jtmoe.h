@@ -105,6 +105,29 @@ int jtmoe_dispatch(const int32_t* expert_ids, const void* x,
                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * jtmoe_dispatch without a workspace argument and without any allocation.  It has no counterpart in
+ * the reference (XLA owns every buffer there and hands the handler its scratch as a result buffer,
+ * rmsnorm_ffi.cu:59-68); it is for callers that cannot allocate device memory at all: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, results and
+ * errors as jtmoe_dispatch; the partial histograms live in a buffer of
+ * JTMOE_DISPATCH_STATIC_MAX_BYTES that is part of the library's device image (each GPU the library
+ * runs on holds its own copy until the process ends).
+ *   Limit: jtmoe_dispatch_workspace_bytes(T*K, E) <= JTMOE_DISPATCH_STATIC_MAX_BYTES, i.e.
+ *   ceil(T*K / 1024) * E <= 262144 (1 048 576 assignments at 256 experts, 4 194 304 at 64);
+ *   beyond it JTMOE_EUNSUPPORTED and nothing is launched.
+ *   All calls on one GPU share that buffer: calls that may overlap on one GPU (two streams, two
+ *   threads) race and must be ordered by the caller.  Nothing in it has to be cleared between
+ *   calls.  The buffer's device address is looked up on the first call per GPU (not a stream
+ *   operation; make that first call outside graph capture).
+ */
+#define JTMOE_DISPATCH_STATIC_MAX_BYTES ((size_t)1 << 20)
+int jtmoe_dispatch_static(const int32_t* expert_ids, const void* x,
+                          int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
+                          int32_t* group_sizes, int32_t* offsets,
+                          int32_t* source_order, int32_t* inverse, void* packed_x,
+                          void* stream);
+
+/*
  * Grouped SwiGLU expert FFN.  Replaces the three jax.lax.ragged_dot calls and
  * the SwiGLU between them (moe.py:638-641):
  *   rows offsets[e] .. offsets[e]+group_sizes[e]-1 of packed_x use expert e;

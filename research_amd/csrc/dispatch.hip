@@ -12,6 +12,8 @@
 // deterministic: no atomics decide a position.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace jtmoe {
 namespace {
 
@@ -298,25 +300,59 @@ extern "C" size_t jtmoe_dispatch_workspace_bytes(int64_t A, int64_t E) {
   return align_up(chunks * (size_t)E * sizeof(int), 256);
 }
 
-extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E, int64_t K,
-                              int dtype, int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
-                              int32_t* inverse, void* packed_x, void* workspace, size_t workspace_bytes,
-                              void* stream) {
-  clear_error();
-  JT_REQUIRE(dtype_ok(dtype), "dispatch: unknown dtype %d", dtype);
-  JT_REQUIRE(T >= 0 && K > 0 && E > 0, "dispatch: T=%lld K=%lld E=%lld out of range", (long long)T, (long long)K,
+namespace jtmoe {
+namespace {
+
+// Scratch of jtmoe_dispatch_static: the partial histograms [E][chunks] of the largest problem it
+// accepts.  Host code must not pass this name to a kernel (on the host it is a stand-in, not a device
+// address): the address on each device comes from hipGetSymbolAddress, once per device.
+constexpr size_t kStaticScratchBytes = JTMOE_DISPATCH_STATIC_MAX_BYTES;  // per GPU, held until the process ends
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices];  // per device, null until looked up
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** out) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+    return fail(JTMOE_ELAUNCH, "dispatch_static: no current device (or its index is beyond %d)", kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr)
+      return fail(JTMOE_ELAUNCH, "dispatch_static: hipGetSymbolAddress failed: %s", hipGetErrorString(err));
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = g_scratch_ptr[device];
+  return JTMOE_OK;
+}
+
+// Argument checks shared by the two entry points (everything but the scratch).
+int dispatch_validate(const char* who, const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E,
+                      int64_t K, int dtype, const int32_t* group_sizes, const int32_t* offsets,
+                      const int32_t* source_order, const int32_t* inverse, const void* packed_x) {
+  JT_REQUIRE(dtype_ok(dtype), "%s: unknown dtype %d", who, dtype);
+  JT_REQUIRE(T >= 0 && K > 0 && E > 0, "%s: T=%lld K=%lld E=%lld out of range", who, (long long)T, (long long)K,
              (long long)E);
-  if (E > JTMOE_MAX_EXPERTS) return fail(JTMOE_EUNSUPPORTED, "dispatch: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  if (E > JTMOE_MAX_EXPERTS) return fail(JTMOE_EUNSUPPORTED, "%s: E=%lld exceeds %d", who, (long long)E, JTMOE_MAX_EXPERTS);
+  JT_REQUIRE(T < ((int64_t)1 << 31) && T * K < ((int64_t)1 << 31), "%s: T*K exceeds int32", who);
+  JT_REQUIRE(group_sizes && offsets, "%s: null pointer argument", who);
+  JT_REQUIRE(T * K == 0 || (expert_ids && source_order && inverse), "%s: null pointer argument", who);
+  JT_REQUIRE(x == nullptr || (H > 0 && packed_x != nullptr), "%s: x given without H or packed_x", who);
+  JT_REQUIRE(x == nullptr || H * (int64_t)dtype_bytes(dtype) < ((int64_t)1 << 31), "%s: row too long", who);
+  return JTMOE_OK;
+}
+
+// The launches of a validated dispatch; `partial` holds jtmoe_dispatch_workspace_bytes(A, E) bytes.
+// Every entry of partial that is read has been written by the histogram pass of the same call, so
+// the scratch needs no clearing between calls.
+int dispatch_launch(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
+                    int32_t* group_sizes, int32_t* offsets, int32_t* source_order, int32_t* inverse, void* packed_x,
+                    int* partial, hipStream_t s) {
   const int64_t A = T * K;
-  JT_REQUIRE(A < ((int64_t)1 << 31), "dispatch: T*K exceeds int32");
-  JT_REQUIRE(group_sizes && offsets && workspace, "dispatch: null pointer argument");
-  JT_REQUIRE(A == 0 || (expert_ids && source_order && inverse), "dispatch: null pointer argument");
-  JT_REQUIRE(x == nullptr || (H > 0 && packed_x != nullptr), "dispatch: x given without H or packed_x");
-  JT_REQUIRE(x == nullptr || H * (int64_t)dtype_bytes(dtype) < ((int64_t)1 << 31), "dispatch: row too long");
-  if (workspace_bytes < jtmoe_dispatch_workspace_bytes(A, E))
-    return fail(JTMOE_EWORKSPACE, "dispatch: workspace %zu < %zu bytes", workspace_bytes,
-                jtmoe_dispatch_workspace_bytes(A, E));
-  hipStream_t s = as_stream(stream);
   if (A > 0 && A <= kSmallMaxAssignments && E <= kSmallMaxExperts) {
     dispatch_small_kernel<<<1, kSmallThreads, (size_t)E * (1 + kSmallWaves) * sizeof(int), s>>>(
         expert_ids, (int)A, (int)E, group_sizes, offsets, source_order, inverse);
@@ -326,7 +362,6 @@ extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t 
     return check_launch("dispatch");
   }
   const int nchunks = dispatch_chunks(A > 0 ? A : 1);
-  int* partial = static_cast<int*>(workspace);
   dispatch_hist_kernel<<<nchunks, kDispThreads, (size_t)E * sizeof(int), s>>>(expert_ids, (int)A, (int)E, nchunks,
                                                                               partial);
   dispatch_scan_kernel<<<1, kScanThreads, 0, s>>>(partial, (int)E, nchunks, group_sizes, offsets);
@@ -339,4 +374,43 @@ extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t 
   if (A == 0) stage_mark(kStageDispatchMeta, s);
   stage_mark(kStageDispatchRows, s);
   return check_launch("dispatch");
+}
+
+}  // namespace
+}  // namespace jtmoe
+
+extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E, int64_t K,
+                              int dtype, int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
+                              int32_t* inverse, void* packed_x, void* workspace, size_t workspace_bytes,
+                              void* stream) {
+  clear_error();
+  const int rc = dispatch_validate("dispatch", expert_ids, x, T, H, E, K, dtype, group_sizes, offsets, source_order,
+                                   inverse, packed_x);
+  if (rc) return rc;
+  JT_REQUIRE(workspace != nullptr, "dispatch: null pointer argument");
+  if (workspace_bytes < jtmoe_dispatch_workspace_bytes(T * K, E))
+    return fail(JTMOE_EWORKSPACE, "dispatch: workspace %zu < %zu bytes", workspace_bytes,
+                jtmoe_dispatch_workspace_bytes(T * K, E));
+  return dispatch_launch(expert_ids, x, T, H, E, K, dtype, group_sizes, offsets, source_order, inverse, packed_x,
+                         static_cast<int*>(workspace), as_stream(stream));
+}
+
+extern "C" int jtmoe_dispatch_static(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E,
+                                     int64_t K, int dtype, int32_t* group_sizes, int32_t* offsets,
+                                     int32_t* source_order, int32_t* inverse, void* packed_x, void* stream) {
+  clear_error();
+  int rc = dispatch_validate("dispatch_static", expert_ids, x, T, H, E, K, dtype, group_sizes, offsets, source_order,
+                             inverse, packed_x);
+  if (rc) return rc;
+  const size_t need = jtmoe_dispatch_workspace_bytes(T * K, E);
+  if (need > kStaticScratchBytes)
+    return fail(JTMOE_EUNSUPPORTED,
+                "dispatch_static: T*K=%lld assignments over E=%lld experts need %zu bytes of scratch, the built-in "
+                "buffer holds %zu (ceil(T*K/1024)*E <= 262144); use jtmoe_dispatch with a workspace",
+                (long long)(T * K), (long long)E, need, kStaticScratchBytes);
+  void* ptr = nullptr;
+  rc = static_scratch(&ptr);
+  if (rc) return rc;
+  return dispatch_launch(expert_ids, x, T, H, E, K, dtype, group_sizes, offsets, source_order, inverse, packed_x,
+                         static_cast<int*>(ptr), as_stream(stream));
 }
