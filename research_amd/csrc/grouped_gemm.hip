@@ -11,6 +11,7 @@
 // bf16, v_mfma_f32_32x32x2_f32 for fp32).
 #include "common.hpp"
 #include "grouped_gemm_dma.hpp"
+#include "grouped_gemm_stream.hpp"
 
 #include <mutex>
 
@@ -198,6 +199,44 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
 }
 
 
+// The stream kernel (grouped_gemm_stream.hpp) for the gate/up launch of the 256-row configurations: the
+// same tiles as one software pipeline through all tiles of a workgroup, results written straight from
+// the accumulators.  Its envelope is narrower than launch_fast's (see stream_ok).
+template <typename Cfg>
+int launch_stream(const void* a, const void* b0, const void* b1, void* c, const int32_t* group_sizes,
+                  const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream,
+                  const int32_t* row_map, int row_div, int64_t a_rows, void* save0, void* save1) {
+  using L = StreamLayout<Cfg>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  auto kernel = &grouped_gemm_stream_kernel<Cfg>;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)L::kSmemBytes);
+  });
+  if (attr_err != hipSuccess)
+    return fail(JTMOE_ELAUNCH, "grouped gemm: kernel set-up: %s", hipGetErrorString(attr_err));
+  const bool dense = group_sizes == nullptr;
+  const int64_t mtiles = dense ? (rows + Cfg::BM - 1) / Cfg::BM : max_m_tiles(rows, E, Cfg::BM);
+  const int64_t nt = (N + Cfg::BN - 1) / Cfg::BN;
+  const int64_t tiles_grid = gemm_grid(mtiles, nt);
+  if (tiles_grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
+  const PersistentSchedule ps = persistent_schedule(tiles_grid, persistent_grid_size(), kTilesPerWorkgroup<Cfg>);
+  kernel<<<(unsigned)ps.grid, Cfg::NT, L::kSmemBytes, stream>>>(
+      static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
+      static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,
+      row_map, row_div, (int)a_rows, static_cast<uint16_t*>(save0), static_cast<uint16_t*>(save1), ps.window, ps.chunk);
+  return JTMOE_OK;
+}
+
+// what the stream kernel needs beyond fast_ok: enough k steps to fill its pipeline, a result below
+// 2^31 bytes (32-bit store offsets) and, with a row map, fewer than 2^27 rows and a divisor of at most 32
+template <typename Cfg>
+inline bool stream_ok(int64_t rows, int64_t Kdim, int64_t N, const int32_t* row_map, int row_div) {
+  return Kdim % Cfg::BK == 0 && Kdim / Cfg::BK >= 2 * Cfg::NSTAGE && rows * N * 2 < ((int64_t)1 << 31) &&
+         (row_map == nullptr || (rows < ((int64_t)1 << 27) && row_div >= 1 && row_div <= 32));
+}
+
 // Mean rows per group below which the 64-row tiles are used.
 constexpr int64_t kSmallGroupRows = 128;
 inline bool small_groups(int64_t rows, int64_t E) { return rows < kSmallGroupRows * E; }
@@ -226,8 +265,11 @@ int launch_pair(const void* x, const void* gate, const void* up, const void* dow
                                               row_div, x_rows, save_gate, save_up)
          : small ? launch_fast<GateUpSmallCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
                                                row_div, x_rows, save_gate, save_up)
-                 : launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
-                                          row_div, x_rows, save_gate, save_up);
+         : stream_ok<GateUpStreamCfg>(rows, H, I, row_map, row_div)
+             ? launch_stream<GateUpStreamCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
+                                              row_div, x_rows, save_gate, save_up)
+             : launch_fast<GateUpCfg>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map,
+                                      row_div, x_rows, save_gate, save_up);
   else
     rc = launch_generic<T, true>(x, gate, up, act, group_sizes, offsets, rows, H, I, E, stream, row_map, row_div,
                                  save_gate, save_up);

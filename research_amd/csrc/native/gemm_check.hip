@@ -8,6 +8,7 @@
 //   gemm_check time       + timing of the library's two configurations at the C3 shape,
 //                           once on N(0,1)-like data and once on all-zero data
 #include "grouped_gemm_bwd.hpp"
+#include "grouped_gemm_stream.hpp"
 
 #include <cmath>
 #include <cstdio>
@@ -123,8 +124,32 @@ static void release(Problem& p) {
 // here), unless g_one_tile_per_workgroup asks for the plain kernel.
 static bool g_one_tile_per_workgroup = false;
 static int g_chunk = -1;  // tiles per workgroup of a persistent launch; -1: as the library chooses
+// the stream kernel (grouped_gemm_stream.hpp): one software pipeline through all tiles of a workgroup
+template <typename Cfg>
+static void launch_stream(Problem& p, bool dense) {
+  using L = StreamLayout<Cfg>;
+  if (p.K / Cfg::BK < 2 * Cfg::NSTAGE) { printf("stream kernel: K too short\n"); exit(1); }
+  const long mt = dense ? (p.rows + Cfg::BM - 1) / Cfg::BM
+                        : (p.rows + Cfg::BM - 1) / Cfg::BM + (p.E < p.rows ? p.E : p.rows);
+  const long nt = (p.N + Cfg::BN - 1) / Cfg::BN;
+  const long tiles_grid = gemm_grid(mt, nt);
+  auto kernel = grouped_gemm_stream_kernel<Cfg>;
+  CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                         (int)L::kSmemBytes));
+  PersistentSchedule ps = persistent_schedule(tiles_grid, 256, g_chunk < 0 ? kTilesPerWorkgroup<Cfg> : g_chunk);
+  if (tiles_grid <= 256) ps = {tiles_grid, 0, 0};
+  kernel<<<(unsigned)ps.grid, Cfg::NT, L::kSmemBytes>>>(
+      p.A, p.B0, Cfg::kDual ? p.B1 : nullptr, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows, p.K,
+      p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, nullptr, nullptr,
+      ps.window, ps.chunk);
+}
+
+static bool g_stream = false;
 template <typename Cfg>
 static void launch(Problem& p, bool dense) {
+  if constexpr (Cfg::BM == 256 && (Cfg::OPT & 128) != 0) {
+    if (g_stream) return launch_stream<Cfg>(p, dense);
+  }
   constexpr bool kCanPersist = Cfg::BM == 256 && Cfg::NSTAGE == 2 && Cfg::BK == 64;
   const bool persist = kCanPersist && !g_one_tile_per_workgroup;
   const long mt = dense ? (p.rows + Cfg::BM - 1) / Cfg::BM
@@ -455,6 +480,9 @@ static void time_decode() {
 
 int main(int argc, char** argv) {
   bool ok = true;
+  // "<mode> nocheck": only the timing mode (for counter collection); otherwise every check runs first
+  const bool nocheck = argc > 2 && !strcmp(argv[2], "nocheck");
+  if (!nocheck) {
   {
     Problem p = make(7, 3001, 576, 392, 1, true, 0, 1.0f);  // ragged groups, N not a multiple of the tile
     ok &= check<GateUpCfg>("gate/up ragged", p);
@@ -561,6 +589,69 @@ int main(int argc, char** argv) {
     ok &= check_tn<WgradCfg>("wgrad 256 unequal groups", w, 0);
     ok &= check_tn<WgradDualCfg>("wgrad dual 256 unequal groups", w, 0);
     release(w);
+  }
+  {
+    // the stream kernel: 32-deep steps with four stages, and 64-deep steps with two
+    g_stream = true;
+    Problem p = make(7, 3001, 576, 392, 51, true, 0, 1.0f);
+    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up ragged", p);
+    ok &= check<DownStream4Cfg>("stream 4 x 32 down ragged", p);
+    ok &= check<GateUpStreamCfg>("stream gate/up ragged", p);
+    ok &= check<DownStreamCfg>("stream down ragged", p);
+    release(p);
+    Problem q = make(5, 2400, 512, 384, 52, true, 3, 1.0f);
+    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up gather on load", q);
+    ok &= check<GateUpStreamCfg>("stream gate/up gather on load", q);
+    release(q);
+    Problem r = make(1, 777, 512, 520, 53, false, 0, 1.0f);
+    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up dense", r, true);
+    ok &= check<DownStream4Cfg>("stream 4 x 32 down dense", r, true);
+    release(r);
+    Problem u = make(40, 70000, 256, 264, 54, true, 0, 1.0f);  // many more tiles than workgroups
+    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up many tiles per workgroup", u);
+    ok &= check<DownStream4Cfg>("stream 4 x 32 down many tiles per workgroup", u);
+    ok &= check<DownStreamCfg>("stream down many tiles per workgroup", u);
+    release(u);
+    Problem v = make(33, 90000, 256, 392, 55, true, 4, 1.0f);  // the same with gathered rows (row map by LDS-DMA)
+    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up many tiles, gather", v);
+    ok &= check<GateUpStreamCfg>("stream gate/up many tiles, gather", v);
+    g_chunk = 0;
+    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up many tiles, gather, one workgroup per CU", v);
+    g_chunk = -1;
+    release(v);
+    g_stream = false;
+  }
+  }  // !nocheck
+  if (ok && argc > 1 && !strcmp(argv[1], "time_stream")) {
+    Problem g = make(64, 131072, 2048, 1408, 4, false, 8, 1.0f);  // rows gathered through a permutation, as in the layer
+    Problem d = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
+    for (int rep = 0; rep < 3; ++rep) {
+      g_stream = false;
+      timeit<GateUpCfg>("gate/up library", g, 20);
+      timeit<DownCfg>("down library", d, 20);
+      g_stream = true;
+      timeit<GateUpStream4Cfg>("gate/up stream 4 x 32", g, 20);
+      timeit<DownStream4Cfg>("down stream 4 x 32", d, 20);
+      timeit<GateUpStreamCfg>("gate/up stream 2 x 64 (library)", g, 20);
+      timeit<DownStreamCfg>("down stream 2 x 64", d, 20);
+      g_chunk = 0;
+      timeit<GateUpStream4Cfg>("gate/up stream 4 x 32, one wg per CU", g, 20);
+      timeit<DownStream4Cfg>("down stream 4 x 32, 4 tiles per wg", d, 20);
+      g_chunk = -1;
+      g_stream = false;
+    }
+    release(g); release(d);
+    // a dense square problem: the steady-state loop without ragged tiles
+    Problem sq = make(1, 8192, 8192, 8192, 6, false, 0, 1.0f);
+    for (int rep = 0; rep < 2; ++rep) {
+      g_stream = false;
+      timeit<DownCfg>("8192^3 library", sq, 10);
+      g_stream = true;
+      timeit<DownStream4Cfg>("8192^3 stream 4 x 32", sq, 10);
+      timeit<DownStreamCfg>("8192^3 stream 2 x 64", sq, 10);
+      g_stream = false;
+    }
+    release(sq);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_unequal_tn")) {
     // weight gradients over groups of very unequal sizes (128 groups, 131072 rows)
