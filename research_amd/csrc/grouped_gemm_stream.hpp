@@ -42,6 +42,14 @@ __device__ __forceinline__ void wait_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// two fp32 values -> their bf16 roundings packed in one dword (lo in the low half): one hardware conversion
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+
 template <typename Cfg>
 struct StreamLayout {
   static constexpr int kRowBufBytes = Cfg::NT * 4;
@@ -247,12 +255,6 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   int cs = 0;  // stage of the current k step
 
   while (true) {
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-      for (int jj = 0; jj < TN; ++jj)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
     const bool wave_has_rows = wm * WM < cur.rows && cur.n0 + wn * Cfg::WNO < N;
     idx += stride;
     --left;
@@ -269,12 +271,17 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
 
     // MFMAs of one 16-deep sub-step on fragment set `cur_set`, interleaved by the scheduler with the
     // LDS reads (two per MFMA) that were written before them
-    auto mfma_substep = [&](int cur_set) {
+    // (`first`: the tile's first sub-step, which accumulates onto zero instead of clearing 128 registers)
+    auto mfma_substep = [&](int cur_set, bool first = false) {
+      f32x16_t zero;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) zero[i] = 0.0f;
 #pragma unroll
       for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
         for (int jj = 0; jj < TN; ++jj)
-          acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[cur_set][jj], af[cur_set][mi], acc[mi][jj], 0, 0, 0);
+          acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[cur_set][jj], af[cur_set][mi],
+                                                                first ? zero : acc[mi][jj], 0, 0, 0);
 #pragma unroll
       for (int g = 0; g < TM * TN; ++g) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -282,11 +289,11 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
       }
     };
     // sub-steps 0 .. KK-2 of a step: fragments of the following sub-step are requested, then this one's MFMAs
-    auto leading_substeps = [&]() {
+    auto leading_substeps = [&](auto first_tag) {
 #pragma unroll
       for (int kk = 0; kk < KK - 1; ++kk) {
         load_frags(cs, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-        mfma_substep(kk & 1);
+        mfma_substep(kk & 1, decltype(first_tag)::value && kk == 0);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
@@ -294,8 +301,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
     // ---- steady part: every step has NS successors inside this tile ----
     int j = 0;
     if (wave_has_rows) {
-      for (; j < nk - NS; ++j) {
-        leading_substeps();
+      auto steady_step = [&](auto first_tag) {
+        leading_substeps(first_tag);
         // the next step's stage has arrived (own loads: the wait; everyone's: the barrier), and every
         // wave holds its last fragments of the current stage, which is therefore free
         wait_and_barrier<(NS - 2) * LPS>();
@@ -320,9 +327,17 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
           __builtin_amdgcn_sched_barrier(0);
         }
         cs = ns;
-      }
+      };
+      steady_step(std::true_type{});  // nk >= 2 NS: the steady part has at least NS steps
+      for (j = 1; j < nk - NS; ++j) steady_step(std::false_type{});
     } else {
       // a tile at the end of a group: this wave's rows lie past it; it only keeps the loads going
+#pragma unroll
+      for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[mi][jj][i] = 0.0f;
       for (; j < nk - NS; ++j) {
         wait_and_barrier<(NS - 2) * LPS>();
         issue(pl, j + NS, cs);
@@ -332,7 +347,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
 
     // ---- last NS steps: requests go to the next tile, if there is one ----
     for (; j < nk; ++j) {
-      if (wave_has_rows) leading_substeps();
+      if (wave_has_rows) leading_substeps(std::false_type{});
       // k steps of this workgroup's stream after this one (only the next tile counts: a load is
       // never issued more than NS <= nk steps ahead)
       const int rem = (nk - 1 - j) + (have_next ? nk : 0);
@@ -390,20 +405,24 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
             unsigned pk[2][2];
 #pragma unroll
             for (int dq = 0; dq < 2; ++dq) {
-              float v[4];
 #pragma unroll
-              for (int t = 0; t < 4; ++t) {
-                const int i = (qq + dq) * 4 + t;
+              for (int tp = 0; tp < 2; ++tp) {  // two neighbouring columns at a time
+                const int i = (qq + dq) * 4 + tp * 2;
                 if (kDual) {
-                  const float g = bf16_round_fast(acc[mi][jj][i]);
-                  const float u = bf16_round_fast(acc[mi][jj + TN / 2][i]);
-                  v[t] = pass == 0 ? silu_rcp(g) * u : (pass == 1 ? g : u);
+                  // both products rounded to bf16 (one packed conversion each), then silu(g) * u on them
+                  const unsigned gb = pack_bf16x2(acc[mi][jj][i], acc[mi][jj][i + 1]);
+                  const unsigned ub = pack_bf16x2(acc[mi][jj + TN / 2][i], acc[mi][jj + TN / 2][i + 1]);
+                  if (pass == 0) {
+                    const float g0 = __uint_as_float(gb << 16), g1 = __uint_as_float(gb & 0xffff0000u);
+                    const float u0 = __uint_as_float(ub << 16), u1 = __uint_as_float(ub & 0xffff0000u);
+                    pk[dq][tp] = pack_bf16x2(silu_rcp(g0) * u0, silu_rcp(g1) * u1);
+                  } else {
+                    pk[dq][tp] = pass == 1 ? gb : ub;
+                  }
                 } else {
-                  v[t] = acc[mi][jj][i];
+                  pk[dq][tp] = pack_bf16x2(acc[mi][jj][i], acc[mi][jj][i + 1]);
                 }
               }
-              pk[dq][0] = (unsigned)bf16_bits_fast(v[0]) | ((unsigned)bf16_bits_fast(v[1]) << 16);
-              pk[dq][1] = (unsigned)bf16_bits_fast(v[2]) | ((unsigned)bf16_bits_fast(v[3]) << 16);
             }
             // before: this lane has columns 8 qq + 4 half + 0..3 (pk[0]) and 8 (qq + 1) + 4 half + 0..3
             // (pk[1]); after: columns 8 (qq + half) + 0..7
@@ -432,16 +451,15 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
 }
 
 // The configuration the library launches for gate/up (routed and shared experts): the tile of GateUpCfg
-// with its 64-deep steps and two stages.  Measured on 64 groups of 2048 gathered rows x 2048 x 1408
-// (alternating in one process): 1.356 ms against 1.402-1.445 ms for grouped_gemm_dma_persistent_kernel
-// and 1.380 ms for 32-deep steps with four stages.
-using GateUpStreamCfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
-// Variants kept for the stand-alone check and its timings: 32-deep steps with four stages, and the
-// down projection's tile (the library keeps grouped_gemm_dma_persistent_kernel for that launch: 128 KB
-// of results per tile go out faster as whole lines through LDS with non-temporal stores,
-// 0.729 against 0.752 ms).
-using GateUpStream4Cfg = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128>;
-using DownStream4Cfg = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768>;
-using DownStreamCfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 128 + 32768>;
+// with 32-deep steps and four stages.  Measured on 64 groups of 2048 gathered rows x 2048 x 1408
+// (alternating in one process): 1.306 ms against 1.400-1.409 ms for grouped_gemm_dma_persistent_kernel
+// and 1.315-1.320 ms for 64-deep steps with two stages.
+using GateUpStreamCfg = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128>;
+// Variants kept for the stand-alone check and its timings: 64-deep steps with two stages, and the
+// down projection's tile (0.725-0.737 ms against 0.723-0.727 ms for grouped_gemm_dma_persistent_kernel,
+// which the library keeps for that launch).
+using GateUpStream2Cfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
+using DownStreamCfg = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768>;
+using DownStream2Cfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 128 + 32768>;
 
 }  // namespace jtmoe

@@ -594,29 +594,29 @@ int main(int argc, char** argv) {
     // the stream kernel: 32-deep steps with four stages, and 64-deep steps with two
     g_stream = true;
     Problem p = make(7, 3001, 576, 392, 51, true, 0, 1.0f);
-    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up ragged", p);
-    ok &= check<DownStream4Cfg>("stream 4 x 32 down ragged", p);
     ok &= check<GateUpStreamCfg>("stream gate/up ragged", p);
     ok &= check<DownStreamCfg>("stream down ragged", p);
+    ok &= check<GateUpStream2Cfg>("stream 2 x 64 gate/up ragged", p);
+    ok &= check<DownStream2Cfg>("stream 2 x 64 down ragged", p);
     release(p);
     Problem q = make(5, 2400, 512, 384, 52, true, 3, 1.0f);
-    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up gather on load", q);
     ok &= check<GateUpStreamCfg>("stream gate/up gather on load", q);
+    ok &= check<GateUpStream2Cfg>("stream 2 x 64 gate/up gather on load", q);
     release(q);
     Problem r = make(1, 777, 512, 520, 53, false, 0, 1.0f);
-    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up dense", r, true);
-    ok &= check<DownStream4Cfg>("stream 4 x 32 down dense", r, true);
+    ok &= check<GateUpStreamCfg>("stream gate/up dense", r, true);
+    ok &= check<DownStreamCfg>("stream down dense", r, true);
     release(r);
     Problem u = make(40, 70000, 256, 264, 54, true, 0, 1.0f);  // many more tiles than workgroups
-    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up many tiles per workgroup", u);
-    ok &= check<DownStream4Cfg>("stream 4 x 32 down many tiles per workgroup", u);
+    ok &= check<GateUpStreamCfg>("stream gate/up many tiles per workgroup", u);
     ok &= check<DownStreamCfg>("stream down many tiles per workgroup", u);
+    ok &= check<DownStream2Cfg>("stream 2 x 64 down many tiles per workgroup", u);
     release(u);
     Problem v = make(33, 90000, 256, 392, 55, true, 4, 1.0f);  // the same with gathered rows (row map by LDS-DMA)
-    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up many tiles, gather", v);
     ok &= check<GateUpStreamCfg>("stream gate/up many tiles, gather", v);
+    ok &= check<GateUpStream2Cfg>("stream 2 x 64 gate/up many tiles, gather", v);
     g_chunk = 0;
-    ok &= check<GateUpStream4Cfg>("stream 4 x 32 gate/up many tiles, gather, one workgroup per CU", v);
+    ok &= check<GateUpStreamCfg>("stream gate/up many tiles, gather, one workgroup per CU", v);
     g_chunk = -1;
     release(v);
     g_stream = false;
@@ -630,13 +630,13 @@ int main(int argc, char** argv) {
       timeit<GateUpCfg>("gate/up library", g, 20);
       timeit<DownCfg>("down library", d, 20);
       g_stream = true;
-      timeit<GateUpStream4Cfg>("gate/up stream 4 x 32", g, 20);
-      timeit<DownStream4Cfg>("down stream 4 x 32", d, 20);
-      timeit<GateUpStreamCfg>("gate/up stream 2 x 64 (library)", g, 20);
-      timeit<DownStreamCfg>("down stream 2 x 64", d, 20);
+      timeit<GateUpStreamCfg>("gate/up stream 4 x 32 (library)", g, 20);
+      timeit<DownStreamCfg>("down stream 4 x 32", d, 20);
+      timeit<GateUpStream2Cfg>("gate/up stream 2 x 64", g, 20);
+      timeit<DownStream2Cfg>("down stream 2 x 64", d, 20);
       g_chunk = 0;
-      timeit<GateUpStream4Cfg>("gate/up stream 4 x 32, one wg per CU", g, 20);
-      timeit<DownStream4Cfg>("down stream 4 x 32, 4 tiles per wg", d, 20);
+      timeit<GateUpStreamCfg>("gate/up stream 4 x 32, one wg per CU", g, 20);
+      timeit<DownStreamCfg>("down stream 4 x 32, 4 tiles per wg", d, 20);
       g_chunk = -1;
       g_stream = false;
     }
@@ -647,8 +647,8 @@ int main(int argc, char** argv) {
       g_stream = false;
       timeit<DownCfg>("8192^3 library", sq, 10);
       g_stream = true;
-      timeit<DownStream4Cfg>("8192^3 stream 4 x 32", sq, 10);
-      timeit<DownStreamCfg>("8192^3 stream 2 x 64", sq, 10);
+      timeit<DownStreamCfg>("8192^3 stream 4 x 32", sq, 10);
+      timeit<DownStream2Cfg>("8192^3 stream 2 x 64", sq, 10);
       g_stream = false;
     }
     release(sq);
