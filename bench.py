@@ -51,26 +51,34 @@ def algorithmic_work(cfg: dict) -> dict:
 
 
 def measured_traffic(config: str, kernel: str):
-    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc summary (None if absent).
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc summary (None if absent), and
+    where that figure comes from.
 
     bench.py cannot read hardware counters itself; profiles/hbm_traffic.json holds the scaled
-    FETCH_SIZE + WRITE_SIZE figures of the same command, and names the command that produced them."""
+    FETCH_SIZE + WRITE_SIZE figures of the same command, names the command that produced them and the
+    source revision of the kernels they were taken on (a schedule change makes them stale)."""
     path = ROOT / "profiles" / "hbm_traffic.json"
     try:
-        return json.loads(path.read_text())[config][kernel]["hbm_bytes_per_launch"]
+        table = json.loads(path.read_text())
+        value = table[config][kernel]["hbm_bytes_per_launch"]
     except (OSError, KeyError, ValueError):
-        return None
+        return None, None
+    return value, {"file": "profiles/hbm_traffic.json", "kernels_at": table.get("_kernels_at"),
+                   "measured_on": table.get("_measured_on")}
 
 
-def cpu_baseline(name: str, sample_tokens: int) -> dict:
+def cpu_baseline(name: str, sample_tokens: int | None) -> dict:
     """The oracle (a NumPy port of the reference layer) timed on the host cores,
-    on the first `sample_tokens` tokens of the same seeded workload."""
+    on the first `sample_tokens` tokens of the same seeded workload (None: all of them)."""
     import numpy as np
 
     from oracle import moe_oracle as O
 
     inp = O.make_inputs(name, seed=0, tokens=sample_tokens)
     cfg = inp["cfg"]
+    whole = sample_tokens is None
+    if whole:
+        sample_tokens = cfg["batch"] * cfg["seq"]
     kwargs = dict(top_k=cfg["K"], route_scale=1.0, dtype=cfg["dtype"], shared=inp["shared"])
     args = (inp["x"], inp["w_router"], inp["expert_bias"], inp["gate"], inp["up"], inp["down"])
     small = inp["x"][:, : min(64, sample_tokens)]
@@ -93,8 +101,9 @@ def cpu_baseline(name: str, sample_tokens: int) -> dict:
         unit="tokens/s",
         cores=cores,
         kind="port",
-        sample=f"first {sample_tokens} tokens of {name} (same seed-0 weights), NumPy oracle with emulated "
-               f"{cfg['dtype']}, one timed call of {dt:.2f} s after a 64-token warm-up call",
+        sample=(f"all {sample_tokens} tokens of {name}" if whole else f"first {sample_tokens} tokens of {name}")
+               + f" (seed-0 weights), NumPy oracle, {'emulated bf16' if cfg['dtype'] == 'bf16' else 'fp32'}, "
+                 f"one timed call of {dt:.2f} s after a 64-token warm-up call",
     )
 
 
@@ -312,6 +321,7 @@ def main() -> int:
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
 
+    traffic, traffic_source = measured_traffic(args.config, "gate_up")
     gate_up_tf = tflops(work["gate_up_flops"], stage_ms["gate_up"])
     active = sum(1 for g in group_sizes if g > 0)
     elem = 2 if cfg["dtype"] == "bf16" else 4
@@ -328,7 +338,8 @@ def main() -> int:
             peak=HBM_PEAK_GBS,
             unit="GB/s",
             frac=gate_up_gbs / HBM_PEAK_GBS,
-            traffic=measured_traffic(args.config, "gate_up"),
+            traffic=traffic,
+            traffic_source=traffic_source,
             avg_launch_ms=stage_ms["gate_up"],
             bytes_per_launch=gate_up_bytes,
         )
@@ -340,7 +351,8 @@ def main() -> int:
             peak=peak,
             unit="TFLOP/s",
             frac=gate_up_tf / peak,
-            traffic=measured_traffic(args.config, "gate_up"),
+            traffic=traffic,
+            traffic_source=traffic_source,
             avg_launch_ms=stage_ms["gate_up"],
             flops_per_launch=work["gate_up_flops"],
         )
@@ -358,6 +370,18 @@ def main() -> int:
         combine_gbs=gbs(work["combine_bytes"], stage_ms["combine"]),
         hbm_peak_gbs=HBM_PEAK_GBS,
     )
+    # the HBM-bound stages as fractions of the 8 TB/s peak (algorithmic bytes / stage time / peak)
+    stages["frac_of_hbm_peak"] = {
+        "router": stages["router_gbs"] / HBM_PEAK_GBS,
+        "dispatch": stages["dispatch_gbs"] / HBM_PEAK_GBS,
+        "dispatch_rows": stages["dispatch_rows_gbs"] / HBM_PEAK_GBS,
+        "combine": stages["combine_gbs"] / HBM_PEAK_GBS,
+    }
+    stages["frac_of_mfma_peak"] = {
+        "gate_up": gate_up_tf / peak,
+        "down": stages["down_tflops"] / peak,
+        "shared": stages["shared_tflops"] / peak,
+    }
 
     line = {
         "metric": "MoE layer tokens/s (64E top-8, d2048); grouped-GEMM MFMA util %",
@@ -394,6 +418,8 @@ def main() -> int:
         line["train"] = train_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, work)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.config, min(args.cpu_sample_tokens, T))
+        # the configuration BASELINE.json names for the CPU (C1: fp32, 2048 tokens, 8 experts), in full
+        line["cpu_baseline_c1"] = cpu_baseline("C1", None)
     print(json.dumps(line))
     return 0
 

@@ -1,8 +1,12 @@
-"""The headline configuration at its full size (C3: 16384 tokens, d_model 2048, 64 experts, top-8,
-d_ff 1408, two shared experts, bf16), checked through properties that do not need a CPU run of the
-whole layer: permutation and histogram invariants, per-token independence against a sub-batch,
-additivity of the shared experts, the oracle on a sample of tokens, and for the backward pass exact
-homogeneity in the cotangent and additivity of the weight gradients over a split of the batch."""
+"""The bf16 configurations at their full sizes -- C2 (8192 tokens, d_model 1024, 16 experts, top-2,
+d_ff 2816), C3 (the headline: 16384 tokens, d_model 2048, 64 experts, top-8, d_ff 1408, two shared
+experts) and C4 (16384 tokens, 128 experts, top-8, d_ff 768, routing skewed by a Zipf expert bias:
+groups of 0 ... ~9950 rows, several experts empty) -- checked through properties that do not need a
+CPU run of the whole layer: permutation and histogram invariants, per-token independence against a
+sub-batch, additivity of the shared experts, the oracle on a sample of tokens, and for the backward
+pass exact homogeneity in the cotangent and additivity of the weight gradients over a split of the
+batch.  The edge patterns of the reference's dispatcher tests (an empty expert, total skew;
+tests/jaxtitan/test_model.py:580-587) appear here at scale in C4."""
 
 from __future__ import annotations
 
@@ -17,18 +21,21 @@ from test_gpu_parity import BF16_MAX_REL, dev, host, rel_err, report
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def c3(gpu):
-    inp = O.make_inputs("C3", seed=0)
+@pytest.fixture(scope="module", params=["C2", "C3", "C4"])
+def c3(request, gpu):
+    """One configuration at full size on the GPU (the fixture keeps the headline's name)."""
+    inp = O.make_inputs(request.param, seed=0)
     cfg = inp["cfg"]
     T = cfg["batch"] * cfg["seq"]
-    d = dict(cfg=cfg, T=T, inp=inp)
+    d = dict(name=request.param, cfg=cfg, T=T, inp=inp)
     d["x"] = dev(inp["x"].reshape(T, cfg["H"]), gpu, "bf16")
     for k in ("w_router", "gate", "up", "down"):
         d[k] = dev(inp[k], gpu, "bf16")
     d["bias"] = dev(inp["expert_bias"], gpu)
-    d["shared"] = tuple(dev(m, gpu, "bf16") for m in inp["shared"])
-    return d
+    d["shared"] = tuple(dev(m, gpu, "bf16") for m in inp["shared"]) if inp["shared"] is not None else None
+    yield d
+    d.clear()
+    torch.cuda.empty_cache()
 
 
 def run(c3, x=None, shared=True):
@@ -57,6 +64,13 @@ def test_full_size_plan_invariants(c3):
     np.testing.assert_allclose(host(r.importance).sum(), w.astype(np.float64).sum(), rtol=1e-5)
     # no token picks an expert twice
     assert np.all(np.diff(np.sort(host(r.expert_ids), axis=1), axis=1) > 0)
+    if c3["name"] == "C4":
+        # the skewed stress case: the six disabled experts (and possibly more) get nothing, a fifth of the
+        # experts take most of the assignments, and the largest group is many tiles tall
+        print(f"[parity] C4 groups: empty={int((sizes == 0).sum())} min_nonempty={int(sizes[sizes > 0].min())} "
+              f"max={int(sizes.max())} top20%_share={np.sort(sizes)[-cfg['E'] // 5:].sum() / A:.3f}", flush=True)
+        assert (sizes == 0).sum() >= 6 and sizes.max() >= 8 * (A // cfg["E"])
+        assert np.sort(sizes)[-cfg["E"] // 5:].sum() >= 0.6 * A
 
 
 def test_full_size_rows_match_sub_batch_and_oracle_sample(c3, gpu):
@@ -77,12 +91,14 @@ def test_full_size_rows_match_sub_batch_and_oracle_sample(c3, gpu):
     ids = host(full.expert_ids)[pick]
     d = O.dispatch(ids, cfg["E"], O.cast_compute(x2, "bf16"))
     packed_y = O.grouped_swiglu(d.packed_x, inp["gate"], inp["up"], inp["down"], d.group_sizes, "bf16")
-    shared_y = O.shared_swiglu(x2, *inp["shared"], "bf16")
+    shared_y = O.shared_swiglu(x2, *inp["shared"], "bf16") if inp["shared"] is not None else None
     want = O.combine(packed_y, d.inverse, host(full.weights)[pick], "bf16", shared_y)
-    assert report("C3 full size, 96 sampled tokens", host(full.y)[pick], want) <= BF16_MAX_REL
+    assert report(f"{c3['name']} full size, 96 sampled tokens", host(full.y)[pick], want) <= BF16_MAX_REL
 
 
 def test_full_size_shared_experts_are_additive(c3):
+    if c3["shared"] is None:
+        pytest.skip("configuration without shared experts")
     with_shared, without = run(c3), run(c3, shared=False)
     assert torch.equal(with_shared.expert_ids, without.expert_ids)
     shared_y = ops.shared_swiglu(c3["x"], *c3["shared"])
@@ -115,5 +131,5 @@ def test_full_size_backward_is_homogeneous_and_additive(c3, gpu):
         total = getattr(ga, name).float() + getattr(gb, name).float()
         ref = getattr(g1, name).float()
         err = float((total - ref).abs().max() / ref.abs().max())
-        print(f"[parity] C3 full size additivity of {name}: max_rel={err:.3e}", flush=True)
+        print(f"[parity] {c3['name']} full size additivity of {name}: max_rel={err:.3e}", flush=True)
         assert err <= BF16_MAX_REL
