@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import torch
 
-from research_amd import grad
+from research_amd import grad, ops
 
 
 class MoeLayerFunction(torch.autograd.Function):
@@ -24,22 +24,34 @@ class MoeLayerFunction(torch.autograd.Function):
         shared = None if shared_gate is None else (shared_gate, shared_up, shared_down)
         result, residuals = grad.moe_forward_train(x, w_router, expert_bias, gate, up, down, top_k, route_scale,
                                                    shared=shared)
-        ctx.result, ctx.residuals = result, residuals
         ctx.route_scale = route_scale
         ctx.has_shared = shared is not None
-        ctx.save_for_backward(x, w_router, gate, up, down, *(shared or ()))
+        # Everything the backward pass reads goes through save_for_backward (which knows how to hold an
+        # output such as the scores without a reference cycle); y itself is not needed again.
+        shared_res = residuals.shared
+        ctx.save_for_backward(x, w_router, gate, up, down, *(shared or ()),
+                              result.expert_ids, result.weights, result.scores, result.group_sizes, result.offsets,
+                              result.source_order, result.inverse, residuals.routed.gate_pre, residuals.routed.up_pre,
+                              *((shared_res.gate_pre, shared_res.up_pre) if shared_res is not None else ()))
         ctx.mark_non_differentiable(result.expert_ids)
         return result.y, result.scores, result.expert_ids
 
     @staticmethod
     def backward(ctx, dy, d_scores, _d_ids):
-        saved = ctx.saved_tensors
+        saved = list(ctx.saved_tensors)
         x, w_router, gate, up, down = saved[:5]
-        shared = tuple(saved[5:8]) if ctx.has_shared else None
+        rest = saved[5:]
+        shared = None
+        if ctx.has_shared:
+            shared, rest = tuple(rest[:3]), rest[3:]
+        ids, weights, scores, group_sizes, offsets, source_order, inverse, gate_pre, up_pre = rest[:9]
+        shared_res = grad.ExpertResiduals(rest[9], rest[10]) if ctx.has_shared else None
+        result = ops.LayerResult(None, ids, weights, scores, None, None, group_sizes, offsets, source_order, inverse)
+        residuals = grad.LayerResiduals(grad.ExpertResiduals(gate_pre, up_pre), shared_res)
         if dy is None:
             dy = torch.zeros_like(x)
         g = grad.moe_backward(x, dy.contiguous(), None if d_scores is None else d_scores.contiguous(), w_router, gate,
-                              up, down, shared, ctx.result, ctx.residuals, ctx.route_scale)
+                              up, down, shared, result, residuals, ctx.route_scale)
         ds = g.d_shared if g.d_shared is not None else (None, None, None)
         return g.dx, g.d_w_router, g.d_gate, g.d_up, g.d_down, ds[0], ds[1], ds[2], None, None, None
 
