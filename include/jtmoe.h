@@ -199,6 +199,18 @@ int jtmoe_sequence_balance_loss(const int32_t* expert_ids, const float* scores,
                                 float* loss, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Gradient of jtmoe_sequence_balance_loss with respect to the scores: what jax.grad yields for
+ * _sequence_balance_loss (moe.py:828-840) when the loss takes part in the training objective.  The
+ * per-sequence counts come from one_hot(expert_ids) (moe.py:832) and carry no gradient.
+ *   d_scores[b,s,e] = g / (B*S) * ( f[b,e] / D - (sum_i f[b,i] * scores[b,s,i]) / D^2 ),
+ *   D = sum_e scores[b,s,e],  f[b,e] = E/(K*S) * #{(s,k): ids[b,s,k]==e},  g = *d_loss (1 if NULL).
+ *   expert_ids [B,S,K] i32; scores [B,S,E] f32; d_loss [1] f32 (device) or NULL; out d_scores [B,S,E] f32.
+ */
+int jtmoe_sequence_balance_loss_backward(const int32_t* expert_ids, const float* scores, const float* d_loss,
+                                         int64_t B, int64_t S, int64_t E, int64_t K,
+                                         float* d_scores, void* stream);
+
+/*
  * SMEBU balancing update: the consumer of expert_counts.  Replaces apply_moe_balance_update
  * (steps/moe_balance.py:97-162) and the bias write of _update_expert_biases (:174-184) for L MoE
  * layers of E experts, on device buffers (hand the layer calls rows of one [L,E] counts buffer as

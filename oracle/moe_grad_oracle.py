@@ -33,6 +33,8 @@ Parity status (exercised in ``tests/test_oracle_grad.py``):
   extra cotangent on the scores.
 * moe_backward: pinned by finite differences of the float64 layer built from the
   three closed forms above with the selection held fixed.
+* sequence_balance_loss_backward: pinned by finite differences of the float64 closed
+  form of the loss with the counts held fixed.
 """
 
 from __future__ import annotations
@@ -161,3 +163,24 @@ def moe_backward(x, w_router, gate, up, down, shared, expert_ids, weights, dy, d
         dx = dx + sg.dx
         d_shared = (sg.d_gate, sg.d_up, sg.d_down)
     return LayerGrad(dx, rg.d_w_router, eg.d_gate, eg.d_up, eg.d_down, d_shared, eg.d_weights)
+
+
+def sequence_balance_loss_backward(expert_ids, scores, top_k, d_loss=1.0) -> np.ndarray:
+    """Gradient with respect to the scores of _sequence_balance_loss (moe.py:828-840):
+    loss = sum_{b,e} f[b,e] * mean_s( scores[b,s,e] / max(sum_e scores[b,s,:], 1e-20) ) / B with
+    f[b,e] = E / (K*S) * count[b,e]; the counts come from one_hot(ids) and carry no gradient.
+    Pinned in tests/test_oracle_grad.py by central finite differences of an independently written
+    float64 forward."""
+    ids = np.asarray(expert_ids)
+    sc = _f64(scores)
+    B, S, E = sc.shape
+    counts = np.zeros((B, E))
+    for b in range(B):
+        counts[b] = np.bincount(ids[b].reshape(-1), minlength=E)[:E]
+    f = counts * (E / (top_k * S))
+    total = sc.sum(-1, keepdims=True)
+    clamped = total <= 1e-20
+    denom = np.where(clamped, 1e-20, total)
+    dot = np.sum(f[:, None, :] * sc, axis=-1, keepdims=True)
+    second = np.where(clamped, 0.0, dot / denom**2)
+    return d_loss / (B * S) * (f[:, None, :] / denom - second)

@@ -60,6 +60,7 @@ PROTOTYPES: dict[str, tuple] = {
     "jtmoe_smebu_update": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_float, c_float, c_float, c_ptr, c_ptr]),
     "jtmoe_balance_workspace_bytes": (c_size, [c_i64, c_i64]),
     "jtmoe_sequence_balance_loss": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
+    "jtmoe_sequence_balance_loss_backward": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr]),
     "jtmoe_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),
     "jtmoe_moe_forward": (
         c_int,

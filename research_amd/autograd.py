@@ -60,3 +60,26 @@ def moe_layer(x, w_router, expert_bias, gate, up, down, top_k, route_scale=1.0, 
     """Differentiable layer on x [T,H]: returns (y [T,H], scores [T,E] float32, expert_ids [T,K] int32)."""
     sg, su, sd = shared if shared is not None else (None, None, None)
     return MoeLayerFunction.apply(x, w_router, gate, up, down, sg, su, sd, expert_bias, top_k, float(route_scale))
+
+
+class SequenceBalanceLossFunction(torch.autograd.Function):
+    """scores [B,S,E] (with expert_ids [B,S,K]) -> the sequence balance loss (moe.py:828-840), differentiable
+    in the scores; the counts derived from the ids are constants."""
+
+    @staticmethod
+    def forward(ctx, scores, expert_ids, top_k):
+        ctx.top_k = top_k
+        ctx.save_for_backward(scores, expert_ids)
+        return ops.sequence_balance_loss(expert_ids, scores, top_k=top_k)
+
+    @staticmethod
+    def backward(ctx, d_loss):
+        scores, expert_ids = ctx.saved_tensors
+        d_scores = ops.sequence_balance_loss_backward(expert_ids, scores, top_k=ctx.top_k,
+                                                      d_loss=d_loss.to(torch.float32).reshape(1).contiguous())
+        return d_scores, None, None
+
+
+def sequence_balance_loss(expert_ids, scores, top_k):
+    """The auxiliary loss as a differentiable function of the router scores [B,S,E]."""
+    return SequenceBalanceLossFunction.apply(scores.contiguous(), expert_ids.contiguous(), int(top_k))

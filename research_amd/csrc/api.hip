@@ -95,6 +95,60 @@ __global__ __launch_bounds__(kBalThreads) void balance_partial_kernel(const int3
   }
 }
 
+// Gradient of the loss with respect to the scores (the counts are piecewise constant and carry none):
+//   d loss / d scores[b,s,e] = g / (B S) * ( f[b,e] / D - (sum_i f[b,i] scores[b,s,i]) / D^2 ),  D = sum_e scores[b,s,e]
+// (for D <= 1e-20, where the forward divides by the constant 1e-20 instead: g / (B S) * f[b,e] / 1e-20).
+// One workgroup per sequence, a wave per token at a time; g is *d_loss, or 1 when d_loss is null.
+__global__ __launch_bounds__(kBalThreads) void balance_backward_kernel(const int32_t* __restrict__ ids,
+                                                                       const float* __restrict__ scores,
+                                                                       const float* __restrict__ d_loss, int B, int S,
+                                                                       int E, int K, float* __restrict__ d_scores) {
+  extern __shared__ float smem[];
+  int* cnt = reinterpret_cast<int*>(smem);  // [E]
+  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int e = tid; e < E; e += kBalThreads) cnt[e] = 0;
+  __syncthreads();
+  const int32_t* ids_b = ids + (size_t)b * S * K;
+  for (int i = tid; i < S * K; i += kBalThreads) {
+    const int id = ids_b[i];
+    if (id >= 0 && id < E) atomicAdd(&cnt[id], 1);
+  }
+  __syncthreads();
+  const float fscale = (float)E / ((float)K * (float)S);
+  const float g = (d_loss ? d_loss[0] : 1.0f) / ((float)B * (float)S);
+  float f[kBalPerLane];
+#pragma unroll
+  for (int j = 0; j < kBalPerLane; ++j) {
+    const int e = lane + j * kWave;
+    f[j] = e < E ? fscale * (float)cnt[e] : 0.0f;
+  }
+  for (int s = wave; s < S; s += kBalWaves) {
+    const size_t row = ((size_t)b * S + s) * E;
+    float v[kBalPerLane];
+    float sum = 0.0f, dot = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kBalPerLane; ++j) {
+      const int e = lane + j * kWave;
+      v[j] = e < E ? scores[row + e] : 0.0f;
+      sum += v[j];
+      dot += f[j] * v[j];
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+      sum += __shfl_xor(sum, m);
+      dot += __shfl_xor(dot, m);
+    }
+    const bool clamped = sum <= 1e-20f;
+    const float d = clamped ? 1e-20f : sum;
+    const float second = clamped ? 0.0f : dot / (d * d);
+#pragma unroll
+    for (int j = 0; j < kBalPerLane; ++j) {
+      const int e = lane + j * kWave;
+      if (e < E) d_scores[row + e] = g * (f[j] / d - second);
+    }
+  }
+}
+
 __global__ void balance_final_kernel(const float* __restrict__ partial, int B, float* __restrict__ loss) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     float t = 0.0f;
@@ -326,6 +380,23 @@ extern "C" int jtmoe_sequence_balance_loss(const int32_t* expert_ids, const floa
   balance_partial_kernel<<<(unsigned)B, kBalThreads, smem, s>>>(expert_ids, scores, (int)S, (int)E, (int)K, partial);
   balance_final_kernel<<<1, 64, 0, s>>>(partial, (int)B, loss);
   return check_launch("sequence_balance_loss");
+}
+
+extern "C" int jtmoe_sequence_balance_loss_backward(const int32_t* expert_ids, const float* scores,
+                                                    const float* d_loss, int64_t B, int64_t S, int64_t E, int64_t K,
+                                                    float* d_scores, void* stream) {
+  clear_error();
+  JT_REQUIRE(B > 0 && S > 0 && E > 0 && K > 0,
+             "sequence_balance_loss_backward: B=%lld S=%lld E=%lld K=%lld out of range", (long long)B, (long long)S,
+             (long long)E, (long long)K);
+  if (E > JTMOE_MAX_EXPERTS)
+    return fail(JTMOE_EUNSUPPORTED, "sequence_balance_loss_backward: E=%lld exceeds %d", (long long)E, JTMOE_MAX_EXPERTS);
+  JT_REQUIRE(B * S * E < ((int64_t)1 << 40) && S * K < ((int64_t)1 << 31) && B < ((int64_t)1 << 24),
+             "sequence_balance_loss_backward: sizes out of range");
+  JT_REQUIRE(expert_ids && scores && d_scores, "sequence_balance_loss_backward: null pointer argument");
+  balance_backward_kernel<<<(unsigned)B, kBalThreads, (size_t)E * sizeof(int), as_stream(stream)>>>(
+      expert_ids, scores, d_loss, (int)B, (int)S, (int)E, (int)K, d_scores);
+  return check_launch("sequence_balance_loss_backward");
 }
 
 extern "C" int jtmoe_router_stats(const float* expert_counts, int64_t E, float* stats6, void* stream) {

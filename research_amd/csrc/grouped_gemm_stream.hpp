@@ -74,6 +74,13 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   using L = StreamLayout<Cfg>;
   static_assert(KK % 2 == 0, "fragment double buffer wants an even number of sub-steps");
   static_assert((Cfg::OPT & 128) != 0, "weight tiles in 4 x 64 blocks");
+  // Timing experiments of the stand-alone check (wrong results by construction, never launched by the
+  // library): OPT & 256 leaves out the operand loads of the steady part of the k loop, OPT & 512 its
+  // fragment reads (the MFMAs then run on the fragments read once before the loop).
+  // OPT & 1024 makes every load of the steady part fetch the tile's first k step again (operands that
+  // are in the nearest cache: the cost of issuing the loads without the memory system behind them).
+  constexpr bool kNoLoads = (Cfg::OPT & 256) != 0, kNoFragReads = (Cfg::OPT & 512) != 0;
+  constexpr bool kSameTile = (Cfg::OPT & 1024) != 0;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -252,6 +259,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   bf16x8_t af[2][TM], bf[2][TN];
   wait_and_barrier<(NS - 1) * LPS>();
   load_frags(0, 0, af[0], bf[0]);
+  if (kNoFragReads) load_frags(0, 1, af[1], bf[1]);
   int cs = 0;  // stage of the current k step
 
   while (true) {
@@ -292,7 +300,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
     auto leading_substeps = [&](auto first_tag) {
 #pragma unroll
       for (int kk = 0; kk < KK - 1; ++kk) {
-        load_frags(cs, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+        if (!kNoFragReads) load_frags(cs, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
         mfma_substep(kk & 1, decltype(first_tag)::value && kk == 0);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -319,8 +327,9 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
           constexpr int kLoadsPer = (LPS + TM * TN - 1) / (TM * TN);
 #pragma unroll
           for (int q = 0; q < kLoadsPer; ++q)
-            if (g * kLoadsPer + q < LPS) issue_one(pl, j + NS, cs, g * kLoadsPer + q);
-          if (g < TM)
+            if (!kNoLoads && g * kLoadsPer + q < LPS) issue_one(pl, kSameTile ? 0 : j + NS, cs, g * kLoadsPer + q);
+          if (kNoFragReads) {
+          } else if (g < TM)
             af[0][g] = load_frag_a(ns, 0, g);
           else if (g < TM + TN)
             bf[0][g - TM] = load_frag_b(ns, 0, g - TM);

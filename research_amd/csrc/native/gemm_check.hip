@@ -653,6 +653,61 @@ int main(int argc, char** argv) {
     }
     release(sq);
   }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_ablation")) {
+    // What bounds the stream kernel: the same launch with parts of the k loop left out (results are
+    // wrong by construction), on N(0,1) x N(0,0.05) operands and on all-zero operands.  Dense problems
+    // (one group), one workgroup per CU.
+    using Full = GateUpStreamCfg;
+    using NoLoads = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 256>;
+    using NoFrags = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 512>;
+    using MfmaOnly = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 256 + 512>;
+    using SqFull = DownStreamCfg;
+    using SqNoLoads = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768 + 256>;
+    using SqNoFrags = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768 + 512>;
+    using SqMfmaOnly = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768 + 256 + 512>;
+    using SameTile = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 1024>;
+    using SqSameTile = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768 + 1024>;
+    g_stream = true;
+    g_chunk = 0;
+    for (float scale : {1.0f, 0.0f}) {
+      printf("-- operand data: %s\n", scale > 0 ? "N(0,1) activations, N(0,0.05) weights" : "all zeros");
+      Problem gd = make(1, 131072, 2048, 1408, 4, false, 0, scale);
+      timeit<Full>("gate/up dense: whole kernel", gd, 10);
+      timeit<NoLoads>("gate/up dense: no operand loads", gd, 10);
+      timeit<NoFrags>("gate/up dense: no fragment reads", gd, 10);
+      timeit<MfmaOnly>("gate/up dense: MFMAs and barriers only", gd, 10);
+      timeit<SameTile>("gate/up dense: loads of one cached k step", gd, 10);
+      release(gd);
+      Problem sq = make(1, 8192, 8192, 8192, 6, false, 0, scale);
+      timeit<SqFull>("8192^3: whole kernel", sq, 10);
+      timeit<SqNoLoads>("8192^3: no operand loads", sq, 10);
+      timeit<SqNoFrags>("8192^3: no fragment reads", sq, 10);
+      timeit<SqMfmaOnly>("8192^3: MFMAs and barriers only", sq, 10);
+      timeit<SqSameTile>("8192^3: loads of one cached k step", sq, 10);
+      release(sq);
+    }
+    g_chunk = -1;
+    g_stream = false;
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "counters_stream")) {
+    // a few launches of each kernel for a hardware-counter run (rocprofv3 --pmc ... -- gemm_check counters_stream nocheck)
+    Problem g = make(64, 131072, 2048, 1408, 4, false, 8, 1.0f);
+    Problem d = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
+    Problem sq = make(1, 8192, 8192, 8192, 6, false, 0, 1.0f);
+    for (int rep = 0; rep < 12; ++rep) {
+      g_stream = false;
+      launch<GateUpCfg>(g, false);
+      launch<DownCfg>(d, false);
+      launch<DownCfg>(sq, false);
+      g_stream = true;
+      launch<GateUpStreamCfg>(g, false);
+      launch<GateUpStream2Cfg>(g, false);
+      launch<DownStreamCfg>(sq, false);
+      g_stream = false;
+    }
+    CK(hipDeviceSynchronize());
+    release(g); release(d); release(sq);
+  }
   if (ok && argc > 1 && !strcmp(argv[1], "time_unequal_tn")) {
     // weight gradients over groups of very unequal sizes (128 groups, 131072 rows)
     const int E = 128, rows = 131072, H = 2048, I = 768;

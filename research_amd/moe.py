@@ -164,9 +164,23 @@ class Param:
         return self._cast
 
 
+_TRUNCATED_NORMAL_STD = 0.87962566103423978  # standard deviation of N(0, 1) truncated to [-2, 2]
+
+
 def lecun_normal(shape: tuple[int, ...], dtype: torch.dtype, device: torch.device, generator: torch.Generator) -> torch.Tensor:
-    fan_in = shape[-2]
-    values = torch.randn(shape, generator=generator, dtype=torch.float32) * (1.0 / math.sqrt(fan_in))
+    """The distribution of the reference's default initialiser, nnx.initializers.lecun_normal()
+    (moe.py:164-167): variance scaling 1 / fan_in with a normal truncated at two standard deviations.
+
+    Axis -2 is the input axis and -1 the output axis; every other axis counts into the receptive field,
+    so for the expert tensors [E, H, I] fan_in = E * H (the product of all axes but the last), as JAX
+    computes it.  Only the distribution can be matched, not JAX's random stream.
+    """
+    fan_in = 1
+    for n in shape[:-1]:
+        fan_in *= int(n)
+    values = torch.empty(shape, dtype=torch.float32)
+    torch.nn.init.trunc_normal_(values, mean=0.0, std=1.0, a=-2.0, b=2.0, generator=generator)
+    values *= math.sqrt(1.0 / max(fan_in, 1)) / _TRUNCATED_NORMAL_STD
     return values.to(dtype).to(device)
 
 

@@ -425,6 +425,28 @@ def sequence_balance_loss(expert_ids: torch.Tensor, scores: torch.Tensor, *, top
     return loss.reshape(())
 
 
+def sequence_balance_loss_backward(expert_ids: torch.Tensor, scores: torch.Tensor, *, top_k: int,
+                                   d_loss: torch.Tensor | None = None) -> torch.Tensor:
+    """Gradient of sequence_balance_loss with respect to the scores [B,S,E] (d_loss: scalar f32 tensor or None = 1)."""
+    if not isinstance(scores, torch.Tensor) or scores.dim() != 3:
+        shape = list(scores.shape) if isinstance(scores, torch.Tensor) else None
+        raise ContractError(f"router scores must have shape [batch, seq, experts], got {shape}")
+    _check(scores, "scores", torch.float32)
+    batch, seq_len, experts = scores.shape
+    _check(expert_ids, "expert_ids", torch.int32, (batch, seq_len, top_k))
+    if d_loss is not None:
+        _check(d_loss, "d_loss", torch.float32)
+        if d_loss.numel() != 1:
+            raise ContractError(f"d_loss must hold one value, got shape {list(d_loss.shape)}")
+    dev = scores.device
+    d_scores = torch.empty_like(scores)
+    status = _lib().jtmoe_sequence_balance_loss_backward(
+        _ptr(expert_ids), _ptr(scores), _ptr(d_loss), batch, seq_len, experts, top_k, _ptr(d_scores), _stream(dev),
+    )
+    _raise(status, "jtmoe_sequence_balance_loss_backward")
+    return d_scores
+
+
 @dataclass
 class LayerResult:
     y: torch.Tensor  # [T,H]

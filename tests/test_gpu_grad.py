@@ -312,3 +312,25 @@ def test_autograd_function_routes_cotangents_to_the_backward_entry(gpu):
     for got, ref in ((x.grad, want.dx), (w.grad, want.d_w_router), (gate.grad, want.d_gate), (up.grad, want.d_up),
                      (down.grad, want.d_down)):
         assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("batch,seq,experts,top_k", [(1, 5, 3, 2), (3, 70, 8, 2), (2, 300, 64, 8), (4, 129, 200, 16)])
+def test_sequence_balance_loss_gradient_matches_oracle(gpu, batch, seq, experts, top_k):
+    """d loss / d scores of the auxiliary loss (moe.py:828-840), alone and through torch autograd."""
+    from research_amd import autograd
+
+    rng = np.random.default_rng(batch * 1000 + seq)
+    scores = (1.0 / (1.0 + np.exp(-rng.standard_normal((batch, seq, experts))))).astype(np.float32)
+    ids = np.stack([[rng.permutation(experts)[:top_k] for _ in range(seq)] for _ in range(batch)]).astype(np.int32)
+    want = G.sequence_balance_loss_backward(ids, scores, top_k, d_loss=1.0)
+    sd, idd = dev(scores, gpu), dev(ids, gpu)
+    got = ops.sequence_balance_loss_backward(idd, sd, top_k=top_k)
+    scale = float(np.max(np.abs(want)))
+    np.testing.assert_allclose(host(got) / scale, want / scale, rtol=1e-4, atol=2e-6)
+    assert torch.equal(got, ops.sequence_balance_loss_backward(idd, sd, top_k=top_k))
+    # through autograd, with a weight on the loss as the training objective applies it
+    s_req = sd.clone().requires_grad_(True)
+    loss = autograd.sequence_balance_loss(idd, s_req, top_k)
+    assert float(loss) == pytest.approx(float(O.sequence_balance_loss(ids, scores, top_k)), rel=1e-5)
+    (g,) = torch.autograd.grad(loss * 0.25, [s_req])
+    np.testing.assert_allclose(host(g) / scale, 0.25 * want / scale, rtol=1e-4, atol=2e-6)

@@ -135,3 +135,24 @@ def test_balance_spec_and_state_contract():
     assert B.router_counts_from_stats((), state).shape == (0, 0)
     with pytest.raises(ContractError, match="MoE balance expected 3 router stat entries, got 2"):
         B.router_counts_from_stats(stats[:2], state)
+
+
+def test_default_initialiser_has_the_reference_distribution():
+    """nnx.initializers.lecun_normal() on [E, H, I]: variance 1 / (E * H), truncated at two standard
+    deviations of the underlying normal (moe.py:164-167; jax.nn.initializers.variance_scaling)."""
+    import math
+
+    import torch
+
+    from research_amd.moe import lecun_normal
+
+    gen = torch.Generator().manual_seed(0)
+    E, H, I = 8, 96, 160
+    w = lecun_normal((E, H, I), torch.float32, torch.device("cpu"), gen)
+    want_std = math.sqrt(1.0 / (E * H))
+    assert abs(float(w.std()) / want_std - 1.0) < 0.02
+    assert abs(float(w.mean())) < 0.02 * want_std
+    assert float(w.abs().max()) <= 2.0 * want_std / 0.87962566103423978 + 1e-9  # the truncation point
+    assert float(w.abs().max()) > 1.9 * want_std / 0.87962566103423978           # and samples reach it
+    k = lecun_normal((H, E), torch.float32, torch.device("cpu"), gen)             # a plain [in, out] kernel
+    assert abs(float(k.std()) / math.sqrt(1.0 / H) - 1.0) < 0.05
