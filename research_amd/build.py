@@ -28,7 +28,7 @@ ARCH = "gfx950"
 SOURCE_FILES = (
     "api.hip", "router.hip", "dispatch.hip", "combine.hip", "norm.hip", "grouped_gemm.hip", "grouped_gemm_bwd.hip",
     "backward.hip", "common.hpp", "gemm_common.hpp", "gemm_launch.hpp", "grouped_gemm_dma.hpp",
-    "grouped_gemm_stream.hpp", "grouped_gemm_bwd.hpp", "native/gemm_check.hip",
+    "grouped_gemm_stream.hpp", "grouped_gemm_bwd.hpp", "dispatch_small.hpp", "native/gemm_check.hip",
 )
 
 

@@ -335,7 +335,7 @@ LayerWorkspace carve_layer(void* base, int64_t T, int64_t H, int64_t E, int64_t 
   LayerWorkspace w;
   w.router_bytes = jtmoe_router_workspace_bytes(E);
   w.router = c.take(w.router_bytes);
-  w.dispatch_bytes = jtmoe_dispatch_workspace_bytes((int64_t)A, E);
+  w.dispatch_bytes = dispatch_layer_workspace_bytes((int64_t)A, E);
   w.dispatch = c.take(w.dispatch_bytes);
   w.packed_x = c.take(A * (size_t)H * b);
   w.act = c.take(A * (size_t)I * b);
@@ -450,8 +450,13 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
   const LayerWorkspace w = carve_layer(workspace, T, H, E, K, I, Is, dtype);
   if (workspace_bytes < w.total)
     return fail(JTMOE_EWORKSPACE, "moe_forward: workspace %zu < %zu bytes", workspace_bytes, w.total);
-  int rc = jtmoe_router(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
-                        expert_counts, importance, nullptr, w.router, w.router_bytes, stream);
+  // The router of a layer call leaves out what the dispatch behind it can do in passing: at large
+  // batches the statistics (no zeroing and no finalising launch, no global atomics), at small ones
+  // its finishing workgroup writes the dispatch plan as well.
+  bool stats_done = false, plan_done = false;
+  int rc = router_for_layer(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
+                            expert_counts, importance, group_sizes, offsets, source_order, inverse, w.router,
+                            w.router_bytes, &stats_done, &plan_done, as_stream(stream));
   if (rc) return rc;
   stage_mark(kStageRouter, as_stream(stream));
   // where the GEMM can apply the permutation while it fetches its A tiles, the permuted copy of
@@ -459,8 +464,9 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
   const bool gather = train || (T > 0 && jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) &&
                       (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(gate) & 15u) == 0 &&
                       (reinterpret_cast<uintptr_t>(up) & 15u) == 0 && (reinterpret_cast<uintptr_t>(down) & 15u) == 0);
-  rc = jtmoe_dispatch(expert_ids, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes, offsets,
-                      source_order, inverse, w.packed_x, w.dispatch, w.dispatch_bytes, stream);
+  rc = dispatch_for_layer(expert_ids, weights, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes,
+                          offsets, source_order, inverse, w.packed_x, expert_counts, importance, w.dispatch,
+                          !stats_done, plan_done, as_stream(stream));
   if (rc) return rc;
   if (train)
     rc = jtmoe_grouped_swiglu_train(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,

@@ -112,4 +112,26 @@ __device__ __forceinline__ void store_stream(V* p, const V& v) {
 void launch_dispatch_rows(const void* x, const int32_t* inverse, int64_t T, int64_t K, int64_t H, int dtype,
                           void* packed_x, hipStream_t stream);
 
+// dispatch.hip: the dispatch as the layer runs it.  want_stats (weights of element type = dtype): the
+// histogram pass also sums the route weights per expert, and expert_counts / importance get the
+// statistics that the router left out (router_for_layer).  The workspace holds
+// dispatch_layer_workspace_bytes(T*K, E) bytes.  plan_done: only the row scatter is left to do.
+size_t dispatch_layer_workspace_bytes(int64_t A, int64_t E);
+int dispatch_for_layer(const int32_t* expert_ids, const void* weights, const void* x, int64_t T, int64_t H, int64_t E,
+                       int64_t K, int dtype, int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
+                       int32_t* inverse, void* packed_x, float* expert_counts, float* importance, void* workspace,
+                       bool want_stats, bool plan_done, hipStream_t stream);
+
+// router.hip: the router as the layer runs it, with the dispatch plan behind it where that is free.
+// On return *stats_done says whether expert_counts / importance have been written (the small-batch
+// path gets them from its one finishing workgroup); if not, the caller's dispatch computes them from
+// the ids and weights.  *plan_done says whether group_sizes / offsets / source_order / inverse have
+// been written as well (the finishing workgroup of the small-batch router goes on to the plan while
+// it still holds the ids in LDS).
+int router_for_layer(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H, int64_t E,
+                     int64_t K, double route_scale, int dtype, int32_t* expert_ids, void* weights, float* scores,
+                     float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
+                     int32_t* source_order, int32_t* inverse, void* workspace, size_t workspace_bytes,
+                     bool* stats_done, bool* plan_done, hipStream_t stream);
+
 }  // namespace jtmoe

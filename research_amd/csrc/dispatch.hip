@@ -11,6 +11,7 @@
 // over (expert-major, chunk-minor) partial histograms, so it is stable and
 // deterministic: no atomics decide a position.
 #include "common.hpp"
+#include "dispatch_small.hpp"
 
 #include <mutex>
 
@@ -25,10 +26,22 @@ constexpr int kDispChunk = kDispThreads * kDispIters;  // assignments per workgr
 inline int dispatch_chunks(int64_t A) { return (int)((A + kDispChunk - 1) / kDispChunk); }
 
 // pass 1: partial[e * nchunks + chunk] = #{a in chunk : ids[a] == e}
-__global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(const int32_t* __restrict__ ids, int A, int E,
-                                                                     int nchunks, int* __restrict__ partial) {
-  extern __shared__ int hist[];
-  for (int e = threadIdx.x; e < E; e += kDispThreads) hist[e] = 0;
+// (kChunkMajor: partial[chunk * E + e], the layout the rank pass reads when it does the scan itself)
+// kStats: also partial_imp[same index] = the sum of the route weights of those assignments,
+// in 32.32 fixed point (the importance of _router_stats, moe.py:804, summed here instead of in the
+// router when the layer runs both)
+template <bool kStats, typename WT, bool kChunkMajor>
+__global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(const int32_t* __restrict__ ids,
+                                                                     const WT* __restrict__ weights, int A, int E,
+                                                                     int nchunks, int* __restrict__ partial,
+                                                                     unsigned long long* __restrict__ partial_imp) {
+  extern __shared__ __align__(8) unsigned char hist_raw[];
+  unsigned long long* const imp = reinterpret_cast<unsigned long long*>(hist_raw);  // [E], kStats only
+  int* const hist = reinterpret_cast<int*>(hist_raw + (kStats ? (size_t)E * 8 : 0));
+  for (int e = threadIdx.x; e < E; e += kDispThreads) {
+    hist[e] = 0;
+    if (kStats) imp[e] = 0ull;
+  }
   __syncthreads();
   const int base = blockIdx.x * kDispChunk;
 #pragma unroll
@@ -36,68 +49,243 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(const int32
     const int a = base + it * kDispThreads + threadIdx.x;
     if (a < A) {
       const int id = ids[a];
-      if (id >= 0 && id < E) atomicAdd(&hist[id], 1);
+      if (id >= 0 && id < E) {
+        atomicAdd(&hist[id], 1);
+        if (kStats) atomicAdd(&imp[id], (unsigned long long)(Elem<WT>::load(weights + a) * kImportanceScale));
+      }
     }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < E; e += kDispThreads) partial[(size_t)e * nchunks + blockIdx.x] = hist[e];
+  for (int e = threadIdx.x; e < E; e += kDispThreads) {
+    const size_t o = kChunkMajor ? (size_t)blockIdx.x * E + e : (size_t)e * nchunks + blockIdx.x;
+    partial[o] = hist[e];
+    if (kStats) partial_imp[o] = imp[e];
+  }
 }
 
-// pass 2 (one workgroup): in-place exclusive scan of partial[0 .. E*nchunks),
-// then group_sizes / offsets per expert.
+// pass 2 (one workgroup of 16 waves): in-place exclusive scan of partial[0 .. E*nchunks), then
+// group_sizes / offsets per expert.  Wave w owns one contiguous segment, which it reads twice with
+// whole-line accesses (64 consecutive ints per step, four steps in flight): once for the segment
+// total, once more to write the running sums.
+// kStats: expert_counts / importance of the layer from the same partial sums.
 constexpr int kScanThreads = 1024;
-__global__ __launch_bounds__(kScanThreads) void dispatch_scan_kernel(int* __restrict__ partial, int E, int nchunks,
+constexpr int kScanWaves = kScanThreads / kWave;
+template <bool kStats>
+__global__ __launch_bounds__(kScanThreads) void dispatch_scan_kernel(int* __restrict__ partial,
+                                                                     const unsigned long long* __restrict__ partial_imp,
+                                                                     int E, int nchunks,
                                                                      int32_t* __restrict__ group_sizes,
-                                                                     int32_t* __restrict__ offsets) {
-  __shared__ int wave_sums[kScanThreads / kWave];
-  __shared__ int total_s;
+                                                                     int32_t* __restrict__ offsets,
+                                                                     float* __restrict__ expert_counts,
+                                                                     float* __restrict__ importance) {
+  __shared__ int wave_total[kScanWaves];
   const int n = E * nchunks;
-  const int per = (n + kScanThreads - 1) / kScanThreads;
-  const int lo = min(n, (int)threadIdx.x * per), hi = min(n, lo + per);
-  int local = 0;
-  for (int i = lo; i < hi; ++i) local += partial[i];
-  // inclusive scan of the 1024 thread sums: inside each wave with shuffles, then over the 16 wave
-  // totals (by every wave for itself), two barriers in all
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  int incl = local;
+  const int seg = (n + kScanWaves * kWave - 1) / (kScanWaves * kWave) * kWave;
+  const int lo = min(n, wave * seg), hi = min(n, lo + seg);
+  int sum = 0;
+  for (int i = lo + lane; i < hi; i += kWave) sum += partial[i];
 #pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const int v = __shfl_up(incl, d);
-    if (lane >= d) incl += v;
-  }
-  if (lane == kWave - 1) wave_sums[wave] = incl;
+  for (int d = kWave / 2; d > 0; d >>= 1) sum += __shfl_xor(sum, d);
+  if (lane == 0) wave_total[wave] = sum;
   __syncthreads();
-  int before = 0;
-  for (int w = 0; w < wave; ++w) before += wave_sums[w];
-  incl += before;
-  int run = incl - local;
-  if (threadIdx.x == kScanThreads - 1) total_s = incl;
-  for (int i = lo; i < hi; ++i) {
-    const int v = partial[i];
-    partial[i] = run;
-    run += v;
+  int carry = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kScanWaves; ++w) {
+    const int v = wave_total[w];
+    if (w < wave) carry += v;
+    total += v;
   }
-  __syncthreads();
-  const int total = total_s;
+  for (int i0 = lo; i0 < hi; i0 += 4 * kWave) {
+    int v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j * kWave + lane;
+      v[j] = i < hi ? partial[i] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j * kWave + lane;
+      int incl = v[j];
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+      }
+      if (i < hi) partial[i] = carry + incl - v[j];
+      carry += __shfl(incl, kWave - 1);
+    }
+  }
+  __syncthreads();  // the running sums written above are read by other threads of the workgroup below
   for (int e = threadIdx.x; e < E; e += kScanThreads) {
     const int start = partial[(size_t)e * nchunks];
     const int next = (e + 1 < E) ? partial[(size_t)(e + 1) * nchunks] : total;
     offsets[e] = start;
     group_sizes[e] = next - start;
+    if (kStats) expert_counts[e] = (float)(next - start);
+  }
+  if (kStats) {
+    // a wave per expert, four experts in flight
+    for (int e0 = wave; e0 < E; e0 += 4 * kScanWaves) {
+      unsigned long long acc[4] = {0ull, 0ull, 0ull, 0ull};
+      for (int c = lane; c < nchunks; c += kWave)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int e = e0 + j * kScanWaves;
+          if (e < E) acc[j] += partial_imp[(size_t)e * nchunks + c];
+        }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) acc[j] += __shfl_xor(acc[j], d);
+        const int e = e0 + j * kScanWaves;
+        if (lane == 0 && e < E) importance[e] = (float)((double)acc[j] * (1.0 / 4294967296.0));
+      }
+    }
+  }
+}
+
+// Up to this many chunks the rank pass works out its bases itself from the chunk-major partial
+// histograms (every workgroup reads all of them, nchunks * E ints) and the scan launch is left out;
+// beyond it that read, which grows with the square of the batch, costs more than the launch.
+constexpr int kDirectMaxChunks = 256;
+
+// LDS of the rank pass: imp[E] of 8 bytes (kDirect && kStats), cursor[E], wavehist[kDispWaves][E],
+// and for kDirect tot[slots], pre[slots], wave_s[kDispWaves] with slots = max(E, kDispThreads)
+inline size_t rank_smem_bytes(int E, bool direct, bool stats) {
+  size_t n = (size_t)E * (1 + kDispWaves) * sizeof(int);
+  if (direct) n += ((size_t)2 * (E > kDispThreads ? E : kDispThreads) + kDispWaves) * sizeof(int);
+  if (direct && stats) n += (size_t)E * 8;
+  return n;
+}
+
+// cursor[e] = (assignments of the experts before e) + (assignments of e in the chunks before this
+// one), from partial[chunk * E + e].  Workgroup 0 also writes the per-expert outputs of the call:
+// offsets, group_sizes and (kStats) expert_counts / importance.
+template <bool kStats>
+__device__ __forceinline__ void chunk_bases(const int* __restrict__ partial,
+                                            const unsigned long long* __restrict__ partial_imp, int E, int nchunks,
+                                            int* cursor, int* tmp, unsigned long long* imp_s,
+                                            int32_t* __restrict__ group_sizes, int32_t* __restrict__ offsets,
+                                            float* __restrict__ expert_counts, float* __restrict__ importance) {
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int slots = E > kDispThreads ? E : kDispThreads;
+  int* const tot_s = tmp;
+  int* const pre_s = tmp + slots;
+  int* const wave_s = pre_s + slots;
+  const bool first = blockIdx.x == 0;
+  if (kStats && first)
+    for (int e = tid; e < E; e += kDispThreads) imp_s[e] = 0ull;
+  if (kStats && first) __syncthreads();
+  // G groups of E threads share out the chunks (chunk c goes to group c % G); with more experts than
+  // threads every thread takes several experts and all chunks
+  const int G = E <= kDispThreads ? kDispThreads / E : 1;
+  for (int e0 = 0; e0 < E; e0 += kDispThreads) {
+    int g = 0, e = e0 + tid;
+    if (E <= kDispThreads) {
+      g = tid / E;
+      e = tid - g * E;
+    }
+    if (g < G && e < E) {
+      int tot = 0, pre = 0;
+      unsigned long long acc = 0ull;
+      // 16 loads in flight at a time: the table is in the L2, what costs is the round trip
+      constexpr int kBatch = 16;
+      for (int c0 = g; c0 < nchunks; c0 += kBatch * G) {
+        int v[kBatch];
+        unsigned long long w[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+          const int c = c0 + j * G;
+          v[j] = c < nchunks ? partial[(size_t)c * E + e] : 0;
+          if (kStats && first) w[j] = c < nchunks ? partial_imp[(size_t)c * E + e] : 0ull;
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+          const int c = c0 + j * G;
+          tot += v[j];
+          pre += c < (int)blockIdx.x ? v[j] : 0;
+          if (kStats && first) acc += w[j];
+        }
+      }
+      tot_s[g * E + e] = tot;
+      pre_s[g * E + e] = pre;
+      if (kStats && first) atomicAdd(&imp_s[e], acc);
+    }
+    if (E <= kDispThreads) break;
+  }
+  __syncthreads();
+  // thread t owns the experts [t * per, t * per + per): their totals, then an exclusive scan over the threads
+  const int per = (E + kDispThreads - 1) / kDispThreads;  // <= 4
+  int tots[4], pres[4], mine = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = tid * per + j;
+    int t = 0, q = 0;
+    if (j < per && e < E) {
+      for (int g = 0; g < G; ++g) {
+        t += tot_s[g * E + e];
+        q += pre_s[g * E + e];
+      }
+    }
+    tots[j] = t;
+    pres[j] = q;
+    mine += t;
+  }
+  int incl = mine;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int v = __shfl_up(incl, d);
+    if (lane >= d) incl += v;
+  }
+  if (lane == kWave - 1) wave_s[wave] = incl;
+  __syncthreads();
+  int run = incl - mine;
+  for (int w = 0; w < wave; ++w) run += wave_s[w];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = tid * per + j;
+    if (j < per && e < E) {
+      cursor[e] = run + pres[j];
+      if (first) {
+        offsets[e] = run;
+        group_sizes[e] = tots[j];
+        if (kStats) {
+          expert_counts[e] = (float)tots[j];
+          importance[e] = (float)((double)imp_s[e] * (1.0 / 4294967296.0));
+        }
+      }
+      run += tots[j];
+    }
   }
 }
 
 // pass 3: stable rank of every assignment inside its chunk + the chunk's base.
+// kDirect: the bases come from chunk_bases (no scan launch before this one); otherwise base_g holds
+// the scanned expert-major table.
+template <bool kDirect, bool kStats>
 __global__ __launch_bounds__(kDispThreads) void dispatch_rank_kernel(const int32_t* __restrict__ ids, int A, int E,
                                                                      int nchunks, const int* __restrict__ base_g,
+                                                                     const unsigned long long* __restrict__ partial_imp,
                                                                      int32_t* __restrict__ source_order,
-                                                                     int32_t* __restrict__ inverse) {
-  extern __shared__ int smem[];
+                                                                     int32_t* __restrict__ inverse,
+                                                                     int32_t* __restrict__ group_sizes,
+                                                                     int32_t* __restrict__ offsets,
+                                                                     float* __restrict__ expert_counts,
+                                                                     float* __restrict__ importance) {
+  extern __shared__ __align__(8) unsigned char rank_raw[];
+  unsigned long long* const imp_s = reinterpret_cast<unsigned long long*>(rank_raw);  // [E], kDirect && kStats
+  int* const smem = reinterpret_cast<int*>(rank_raw + ((kDirect && kStats) ? (size_t)E * 8 : 0));
   int* cursor = smem;         // [E] next free packed row of expert e for this chunk
   int* wavehist = smem + E;   // [kDispWaves][E]
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  for (int e = tid; e < E; e += kDispThreads) cursor[e] = base_g[(size_t)e * nchunks + blockIdx.x];
   for (int i = tid; i < kDispWaves * E; i += kDispThreads) wavehist[i] = 0;
+  if (kDirect) {
+    chunk_bases<kStats>(base_g, partial_imp, E, nchunks, cursor, wavehist + kDispWaves * E, imp_s, group_sizes,
+                        offsets, expert_counts, importance);
+  } else {
+    for (int e = tid; e < E; e += kDispThreads) cursor[e] = base_g[(size_t)e * nchunks + blockIdx.x];
+  }
   __syncthreads();
   int nbits = 0;
   while ((1 << nbits) < E) ++nbits;
@@ -143,90 +331,22 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_rank_kernel(const int32
   }
 }
 
-// Small batches: the three passes in one workgroup of 1024 threads (histogram in LDS, scan over the
-// experts with wave shuffles, then the same ballot ranking with 16 waves per round of 1024
-// assignments).  At a few hundred assignments the three launches above are idle most of their
-// time; this is one launch with the same results.
+// Small batches: the three passes in one workgroup of 1024 threads (dispatch_small.hpp).  At a few
+// hundred assignments the three launches above are idle most of their time; this is one launch with
+// the same results.
 constexpr int kSmallThreads = 1024;
-constexpr int kSmallWaves = kSmallThreads / kWave;
-constexpr int kSmallMaxAssignments = 8192;
-constexpr int kSmallMaxExperts = JTMOE_MAX_EXPERTS;  // one thread per expert in the scan
-__global__ __launch_bounds__(kSmallThreads) void dispatch_small_kernel(const int32_t* __restrict__ ids, int A, int E,
+template <bool kStats, typename WT>
+__global__ __launch_bounds__(kSmallThreads) void dispatch_small_kernel(const int32_t* __restrict__ ids,
+                                                                      const WT* __restrict__ weights, int A, int E,
                                                                       int32_t* __restrict__ group_sizes,
                                                                       int32_t* __restrict__ offsets,
                                                                       int32_t* __restrict__ source_order,
-                                                                      int32_t* __restrict__ inverse) {
-  extern __shared__ int smem[];
-  int* cursor = smem;        // [E] histogram, then the next free packed row of expert e
-  int* wavehist = smem + E;  // [kSmallWaves][E]
-  __shared__ int wave_sums[kSmallWaves];
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  for (int e = tid; e < E; e += kSmallThreads) cursor[e] = 0;
-  for (int i = tid; i < kSmallWaves * E; i += kSmallThreads) wavehist[i] = 0;
-  __syncthreads();
-  for (int a = tid; a < A; a += kSmallThreads) {
-    const int id = ids[a];
-    if (id >= 0 && id < E) atomicAdd(&cursor[id], 1);
-  }
-  __syncthreads();
-  // exclusive scan over the experts: thread e owns expert e (E <= 1024 threads)
-  const int count = tid < E ? cursor[tid] : 0;
-  int incl = count;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const int v = __shfl_up(incl, d);
-    if (lane >= d) incl += v;
-  }
-  if (lane == kWave - 1) wave_sums[wave] = incl;
-  __syncthreads();
-  int before = 0;
-  for (int w = 0; w < wave; ++w) before += wave_sums[w];
-  const int start = incl + before - count;
-  if (tid < E) {
-    offsets[tid] = start;
-    group_sizes[tid] = count;
-    cursor[tid] = start;
-  }
-  __syncthreads();
-  int nbits = 0;
-  while ((1 << nbits) < E) ++nbits;
-  for (int base = 0; base < A; base += kSmallThreads) {
-    const int a = base + tid;
-    int id = -1;
-    if (a < A) {
-      id = ids[a];
-      if (id < 0 || id >= E) id = -1;
-    }
-    const bool valid = id >= 0;
-    unsigned long long peers = __ballot(valid);  // lanes of this wave holding the same expert id
-    for (int b = 0; b < nbits; ++b) {
-      const bool bit = (id >> b) & 1;
-      const unsigned long long m = __ballot(valid && bit);
-      peers &= bit ? m : ~m;
-    }
-    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
-    if (valid && rank == 0) wavehist[wave * E + id] = __popcll(peers);
-    __syncthreads();
-    if (valid) {
-      int pos = cursor[id] + rank;
-      for (int w = 0; w < wave; ++w) pos += wavehist[w * E + id];
-      inverse[a] = pos;
-      source_order[pos] = a;
-    } else if (a < A) {
-      inverse[a] = -1;
-    }
-    __syncthreads();
-    for (int e = tid; e < E; e += kSmallThreads) {
-      int add = 0;
-#pragma unroll
-      for (int w = 0; w < kSmallWaves; ++w) {
-        add += wavehist[w * E + e];
-        wavehist[w * E + e] = 0;
-      }
-      cursor[e] += add;
-    }
-    __syncthreads();
-  }
+                                                                      int32_t* __restrict__ inverse,
+                                                                      float* __restrict__ expert_counts,
+                                                                      float* __restrict__ importance) {
+  extern __shared__ __align__(8) unsigned char small_raw[];
+  dispatch_small_body<kSmallThreads, kStats, WT>(ids, weights, A, E, group_sizes, offsets, source_order, inverse,
+                                                 expert_counts, importance, small_raw);
 }
 
 // pass 4: token-major row scatter; each token row is read once and written to
@@ -346,28 +466,73 @@ int dispatch_validate(const char* who, const int32_t* expert_ids, const void* x,
   return JTMOE_OK;
 }
 
-// The launches of a validated dispatch; `partial` holds jtmoe_dispatch_workspace_bytes(A, E) bytes.
+// Where the fixed-point weight sums [E][chunks] of the layer's statistics start inside the scratch.
+inline size_t partial_imp_offset(int64_t A, int64_t E) { return jtmoe_dispatch_workspace_bytes(A, E); }
+
+// The launches of a validated dispatch; `partial` holds jtmoe_dispatch_workspace_bytes(A, E) bytes
+// (dispatch_layer_workspace_bytes(A, E) when `weights` is given).
 // Every entry of partial that is read has been written by the histogram pass of the same call, so
 // the scratch needs no clearing between calls.
-int dispatch_launch(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
-                    int32_t* group_sizes, int32_t* offsets, int32_t* source_order, int32_t* inverse, void* packed_x,
-                    int* partial, hipStream_t s) {
+// stats (weights of element type = dtype): also expert_counts[E] and importance[E], the statistics
+// that jtmoe_router would have produced for these ids and weights.
+template <typename WT>
+int dispatch_launch_t(const int32_t* expert_ids, const WT* weights, bool stats, const void* x, int64_t T, int64_t H,
+                      int64_t E, int64_t K, int dtype, int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
+                      int32_t* inverse, void* packed_x, float* expert_counts, float* importance, int* partial,
+                      hipStream_t s) {
   const int64_t A = T * K;
   if (A > 0 && A <= kSmallMaxAssignments && E <= kSmallMaxExperts) {
-    dispatch_small_kernel<<<1, kSmallThreads, (size_t)E * (1 + kSmallWaves) * sizeof(int), s>>>(
-        expert_ids, (int)A, (int)E, group_sizes, offsets, source_order, inverse);
+    const size_t smem = dispatch_small_smem_bytes((int)E, kSmallThreads, stats);
+    if (stats)
+      dispatch_small_kernel<true, WT><<<1, kSmallThreads, smem, s>>>(expert_ids, weights, (int)A, (int)E, group_sizes,
+                                                                     offsets, source_order, inverse, expert_counts,
+                                                                     importance);
+    else
+      dispatch_small_kernel<false, WT><<<1, kSmallThreads, smem, s>>>(expert_ids, nullptr, (int)A, (int)E, group_sizes,
+                                                                      offsets, source_order, inverse, nullptr, nullptr);
     stage_mark(kStageDispatchMeta, s);
     if (x != nullptr) launch_dispatch_rows(x, inverse, T, K, H, dtype, packed_x, s);
     stage_mark(kStageDispatchRows, s);
     return check_launch("dispatch");
   }
   const int nchunks = dispatch_chunks(A > 0 ? A : 1);
-  dispatch_hist_kernel<<<nchunks, kDispThreads, (size_t)E * sizeof(int), s>>>(expert_ids, (int)A, (int)E, nchunks,
-                                                                              partial);
-  dispatch_scan_kernel<<<1, kScanThreads, 0, s>>>(partial, (int)E, nchunks, group_sizes, offsets);
+  unsigned long long* const partial_imp =
+      stats ? reinterpret_cast<unsigned long long*>(reinterpret_cast<unsigned char*>(partial) + partial_imp_offset(A, E))
+            : nullptr;
+  // two launches (histogram, rank with its own scan) up to kDirectMaxChunks chunks, three beyond
+  const bool direct = A > 0 && nchunks <= kDirectMaxChunks;
+  const size_t hist_smem = (size_t)E * (stats ? 12 : 4);
+#define JT_HIST(STATS, DIRECT)                                                                             \
+  dispatch_hist_kernel<STATS, WT, DIRECT><<<nchunks, kDispThreads, hist_smem, s>>>(expert_ids, weights, (int)A, \
+                                                                                   (int)E, nchunks, partial,    \
+                                                                                   partial_imp)
+#define JT_RANK(DIRECT, STATS)                                                                                  \
+  dispatch_rank_kernel<DIRECT, STATS><<<nchunks, kDispThreads, rank_smem_bytes((int)E, DIRECT, STATS), s>>>(    \
+      expert_ids, (int)A, (int)E, nchunks, partial, partial_imp, source_order, inverse, group_sizes, offsets,   \
+      expert_counts, importance)
+  if (direct) {
+    if (stats) {
+      JT_HIST(true, true);
+      JT_RANK(true, true);
+    } else {
+      JT_HIST(false, true);
+      JT_RANK(true, false);
+    }
+  } else {
+    if (stats) {
+      JT_HIST(true, false);
+      dispatch_scan_kernel<true><<<1, kScanThreads, 0, s>>>(partial, partial_imp, (int)E, nchunks, group_sizes, offsets,
+                                                            expert_counts, importance);
+    } else {
+      JT_HIST(false, false);
+      dispatch_scan_kernel<false><<<1, kScanThreads, 0, s>>>(partial, nullptr, (int)E, nchunks, group_sizes, offsets,
+                                                             nullptr, nullptr);
+    }
+    if (A > 0) JT_RANK(false, false);
+  }
+#undef JT_HIST
+#undef JT_RANK
   if (A > 0) {
-    dispatch_rank_kernel<<<nchunks, kDispThreads, (size_t)E * (1 + kDispWaves) * sizeof(int), s>>>(
-        expert_ids, (int)A, (int)E, nchunks, partial, source_order, inverse);
     stage_mark(kStageDispatchMeta, s);
     if (x != nullptr) launch_dispatch_rows(x, inverse, T, K, H, dtype, packed_x, s);
   }
@@ -376,7 +541,45 @@ int dispatch_launch(const int32_t* expert_ids, const void* x, int64_t T, int64_t
   return check_launch("dispatch");
 }
 
+int dispatch_launch(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
+                    int32_t* group_sizes, int32_t* offsets, int32_t* source_order, int32_t* inverse, void* packed_x,
+                    int* partial, hipStream_t s) {
+  return dispatch_launch_t<float>(expert_ids, nullptr, false, x, T, H, E, K, dtype, group_sizes, offsets, source_order,
+                                  inverse, packed_x, nullptr, nullptr, partial, s);
+}
+
 }  // namespace
+
+size_t dispatch_layer_workspace_bytes(int64_t A, int64_t E) {
+  if (A < 0 || E <= 0) return 0;
+  const size_t chunks = (size_t)dispatch_chunks(A > 0 ? A : 1);
+  return jtmoe_dispatch_workspace_bytes(A, E) + align_up(chunks * (size_t)E * sizeof(unsigned long long), 256);
+}
+
+int dispatch_for_layer(const int32_t* expert_ids, const void* weights, const void* x, int64_t T, int64_t H, int64_t E,
+                       int64_t K, int dtype, int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
+                       int32_t* inverse, void* packed_x, float* expert_counts, float* importance, void* workspace,
+                       bool want_stats, bool plan_done, hipStream_t s) {
+  const int rc = dispatch_validate("dispatch", expert_ids, x, T, H, E, K, dtype, group_sizes, offsets, source_order,
+                                   inverse, packed_x);
+  if (rc) return rc;
+  JT_REQUIRE(workspace != nullptr, "dispatch: null pointer argument");
+  JT_REQUIRE(!want_stats || (expert_counts && importance && (weights || T == 0)), "dispatch: null pointer argument");
+  if (plan_done) {  // the router's finishing workgroup has written the plan
+    stage_mark(kStageDispatchMeta, s);
+    if (x != nullptr && T > 0) launch_dispatch_rows(x, inverse, T, K, H, dtype, packed_x, s);
+    stage_mark(kStageDispatchRows, s);
+    return check_launch("dispatch");
+  }
+  if (dtype == JTMOE_BF16)
+    return dispatch_launch_t<bf16_raw>(expert_ids, static_cast<const bf16_raw*>(weights), want_stats, x, T, H, E, K,
+                                       dtype, group_sizes, offsets, source_order, inverse, packed_x, expert_counts,
+                                       importance, static_cast<int*>(workspace), s);
+  return dispatch_launch_t<float>(expert_ids, static_cast<const float*>(weights), want_stats, x, T, H, E, K, dtype,
+                                  group_sizes, offsets, source_order, inverse, packed_x, expert_counts, importance,
+                                  static_cast<int*>(workspace), s);
+}
+
 }  // namespace jtmoe
 
 extern "C" int jtmoe_dispatch(const int32_t* expert_ids, const void* x, int64_t T, int64_t H, int64_t E, int64_t K,

@@ -9,6 +9,7 @@
 // IEEE-754 single operations, so the routing decision is a pure function of the
 // logits and can be reproduced bit for bit on a CPU.
 #include "common.hpp"
+#include "dispatch_small.hpp"
 
 #include <mutex>
 
@@ -17,7 +18,7 @@ namespace {
 
 // A workgroup of NW waves routes 16*NW tokens with 64*NW threads (4 lanes per token in the
 // selection phase).
-constexpr float kFixedScale = 4294967296.0f;  // importance is summed in 32.32 fixed point
+constexpr float kFixedScale = kImportanceScale;  // importance is summed in 32.32 fixed point
 
 // ---- fully specified fp32 sigmoid ------------------------------------------
 __device__ __forceinline__ float exp_fixed(float x) {
@@ -59,9 +60,9 @@ struct RouterScratch {
 };
 
 __host__ __device__ inline RouterScratch router_scratch(void* ws, int E) {
-  RouterScratch s;
+  RouterScratch s;  // ws == null: a call that leaves the statistics to the dispatch behind it
   s.imp = reinterpret_cast<unsigned long long*>(ws);
-  s.cnt = reinterpret_cast<int*>(s.imp + E);
+  s.cnt = ws ? reinterpret_cast<int*>(s.imp + E) : nullptr;
   return s;
 }
 
@@ -292,6 +293,7 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
     }
     return;
   }
+  if (g.cnt == nullptr) return;
   for (int e = tid; e < E; e += kRouterThreads) {
     const int c = sm.cnt[e];
     if (c) {
@@ -384,8 +386,14 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
   // Loads run D chunks ahead of the MFMAs through a ring of registers (chunk c lives in slot
   // c % D), so that the latency of a load is hidden by D - 1 whole iterations instead of by the
   // few MFMAs of one: with a single chunk in flight every iteration waits for memory.
-  constexpr int D = CW <= 8 ? 3 : (CW <= 16 ? 2 : 1);
-  constexpr int UNROLL = D == 3 ? 6 : 2;  // a multiple of D and of the two LDS stages
+  // The memory pipeline returns loads in order, so what is in flight while a wave waits for the
+  // next chunk of the router matrix is everything issued after it: D - 1 chunks of the matrix and of
+  // x.  x comes from HBM (the only large stream of this kernel, 2 KB per wave and chunk): with three
+  // slots a CU had 16 KB of it in flight and the kernel ran at a quarter of the HBM rate; the ring
+  // is as deep as the registers of the matrix chunks allow.
+  constexpr int D = CW <= 2 ? 8 : (CW <= 4 ? 6 : (CW <= 8 ? 4 : 2));
+  constexpr int UNROLL = D;  // a multiple of D and of the two LDS stages
+  static_assert(D % 2 == 0, "the unrolled body alternates between the two LDS stages");
   u32x4_t a_ring[D][2], w_ring[D][CW];
   f32x4_t acc[NB];
 #pragma unroll
@@ -642,12 +650,19 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
 // Second half of the small-batch router: one workgroup adds the slices of partial sums in slice
 // order, rounds to bf16 (the projection's output dtype) and runs the epilogue for every token of
 // the call, so the statistics need neither the zeroing nor the finalising launch.
-constexpr int kPartialMaxSlices = 16;
-template <int kTok>
+//
+// kPlan: the workgroup then goes on to the dispatch plan of these assignments (group sizes, offsets,
+// the stable permutation and its inverse) from the ids it holds in LDS; the tables of that step take
+// the place of the score tile, which is dead by then.  Requires tokens * K <= kSmallMaxAssignments
+// and E <= 4 * kTok.
+constexpr int kPartialMaxSlices = 8;
+template <int kTok, bool kPlan>
 __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
     const float* __restrict__ partial, int slices, const float* __restrict__ bias, int tokens, int E, int K,
     float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights, float* __restrict__ scores,
-    float* __restrict__ logits_out, float* __restrict__ counts, float* __restrict__ importance) {
+    float* __restrict__ logits_out, float* __restrict__ counts, float* __restrict__ importance,
+    int32_t* __restrict__ group_sizes, int32_t* __restrict__ offsets, int32_t* __restrict__ source_order,
+    int32_t* __restrict__ inverse) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   RouterSmem sm = router_smem(smem_raw, E, K, kTok);
   const int stride = E + 1;
@@ -667,6 +682,12 @@ __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
   __syncthreads();
   router_epilogue<bf16_raw, kTok, 4 * kTok>(sm, bias, 0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
                                             RouterScratch{}, counts, importance);
+  if (kPlan) {
+    static_assert(kTok >= 1 + 4 * kTok / kWave, "the plan's tables fit into the score tile");
+    dispatch_small_body<4 * kTok, false, bf16_raw>(sm.top_id, nullptr, tokens * K, E, group_sizes, offsets,
+                                                   source_order, inverse, nullptr, nullptr,
+                                                   reinterpret_cast<unsigned char*>(sm.tile));
+  }
 }
 
 template <typename KernelT>
@@ -678,11 +699,26 @@ int set_max_smem(KernelT kernel, size_t bytes) {
   return JTMOE_OK;
 }
 
+// What a layer call adds to a router call: it may leave the statistics to the dispatch that follows
+// (stats_done = false on return), and the small-batch path writes the dispatch plan as well.
+struct LayerPlan {
+  int32_t* group_sizes;
+  int32_t* offsets;
+  int32_t* source_order;
+  int32_t* inverse;
+  bool stats_done;
+  bool plan_done;
+};
+
 template <typename T, bool kFromLogits>
 int launch_router(const void* x, const void* w, const float* logits_in, const float* bias, int64_t tokens,
                   int64_t H, int64_t E, int64_t K, double route_scale, int32_t* ids, void* weights,
                   float* scores, float* counts, float* importance, float* logits_out, void* ws,
-                  hipStream_t stream) {
+                  hipStream_t stream, LayerPlan* layer = nullptr) {
+  // a stand-alone call always computes the statistics; a layer call only where they cost no launch
+  const bool stats = layer == nullptr;
+  void* const ws_stats = stats ? ws : nullptr;
+  if (layer) layer->stats_done = layer->plan_done = false;
   const bool mfma = Elem<T>::is_bf16 && !kFromLogits && H % kRouterKC == 0 && H * E < ((int64_t)1 << 30) &&
                     (E == 16 || E == 32 || E == 64 || E == 128 || E == 256) && aligned16(x) && aligned16(w);
   if (mfma) {
@@ -721,22 +757,31 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
         }
 #undef JT_PARTIAL_CASE
         const size_t fsmem = router_smem_bytes((int)E, (int)K, finish_tok);
+        const bool plan = layer != nullptr && tokens * K <= kSmallMaxAssignments && E <= 4 * finish_tok;
+#define JT_FINISH(TOK, PLAN)                                                                                       \
+  {                                                                                                                \
+    auto kernel = router_finish_kernel<TOK, PLAN>;                                                                 \
+    int rc = set_max_smem(kernel, fsmem);                                                                          \
+    if (rc) return rc;                                                                                             \
+    kernel<<<1, 4 * TOK, fsmem, stream>>>(partial, slices, bias, (int)tokens, (int)E, (int)K, (float)route_scale,  \
+                                          ids, static_cast<bf16_raw*>(weights), scores, logits_out, counts,        \
+                                          importance, PLAN ? layer->group_sizes : nullptr,                         \
+                                          PLAN ? layer->offsets : nullptr, PLAN ? layer->source_order : nullptr,   \
+                                          PLAN ? layer->inverse : nullptr);                                        \
+  }
         if (finish_tok == 256) {
-          auto kernel = router_finish_kernel<256>;
-          int rc = set_max_smem(kernel, fsmem);
-          if (rc) return rc;
-          kernel<<<1, 1024, fsmem, stream>>>(partial, slices, bias, (int)tokens, (int)E, (int)K, (float)route_scale, ids,
-                                             static_cast<bf16_raw*>(weights), scores, logits_out, counts, importance);
+          if (plan) JT_FINISH(256, true) else JT_FINISH(256, false)
         } else {
-          auto kernel = router_finish_kernel<64>;
-          int rc = set_max_smem(kernel, fsmem);
-          if (rc) return rc;
-          kernel<<<1, 256, fsmem, stream>>>(partial, slices, bias, (int)tokens, (int)E, (int)K, (float)route_scale, ids,
-                                            static_cast<bf16_raw*>(weights), scores, logits_out, counts, importance);
+          if (plan) JT_FINISH(64, true) else JT_FINISH(64, false)
+        }
+#undef JT_FINISH
+        if (layer) {
+          layer->stats_done = true;
+          layer->plan_done = plan;
         }
         return check_launch("router");
       }
-      router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
+      if (stats) router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
       if (tokens > 0) {
 #define JT_SPLIT_CASE(NB)                                                                                     \
   case NB * 16: {                                                                                            \
@@ -745,7 +790,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (rc) return rc;                                                                                       \
     kernel<<<blocks, 256, smem, stream>>>(                                                                   \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws, nullptr, 0);       \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats, nullptr, 0); \
   } break;
         switch ((int)E) {
           JT_SPLIT_CASE(1)
@@ -756,7 +801,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
         }
 #undef JT_SPLIT_CASE
       }
-      router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
+      if (stats) router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
       return check_launch("router");
     }
     // four waves (64 tokens) per workgroup: the waves share the work of bringing in the router
@@ -766,7 +811,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     const int blocks = (int)((tokens + tok - 1) / tok);
     const size_t smem = router_mfma_smem_bytes((int)E, (int)K, tok);
     if (smem > 160 * 1024) return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
-    router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
+    if (stats) router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
     if (tokens > 0) {
 #define JT_ROUTER_LAUNCH(NB, NW)                                                                             \
   {                                                                                                          \
@@ -775,7 +820,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (rc) return rc;                                                                                       \
     kernel<<<blocks, 64 * NW, smem, stream>>>(                                                               \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws);                   \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats);             \
   }
 #define JT_ROUTER_CASE(NB)    \
   case NB * 16:               \
@@ -798,13 +843,13 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     auto kernel = router_kernel<T, kFromLogits>;
     int rc = set_max_smem(kernel, smem);
     if (rc) return rc;
-    router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
+    if (stats) router_zero_kernel<<<1, 256, 0, stream>>>(ws, (int)E);
     if (tokens > 0)
       kernel<<<blocks, 256, smem, stream>>>(
           static_cast<const T*>(x), static_cast<const T*>(w), logits_in, bias, (int)tokens, (int)H, (int)E, (int)K,
-          (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws);
+          (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws_stats);
   }
-  router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
+  if (stats) router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
   return check_launch("router");
 }
 
@@ -822,6 +867,31 @@ int validate_router(int64_t T, int64_t H, int64_t E, int64_t K, double route_sca
 }
 
 }  // namespace
+
+int router_for_layer(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H, int64_t E,
+                     int64_t K, double route_scale, int dtype, int32_t* expert_ids, void* weights, float* scores,
+                     float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
+                     int32_t* source_order, int32_t* inverse, void* workspace, size_t workspace_bytes,
+                     bool* stats_done, bool* plan_done, hipStream_t s) {
+  int rc = validate_router(T, H, E, K, route_scale, dtype, true);
+  if (rc) return rc;
+  JT_REQUIRE(w_router && expert_counts && importance && workspace, "router: null pointer argument");
+  JT_REQUIRE(T == 0 || (x && expert_ids && weights && scores), "router: null pointer argument");
+  JT_REQUIRE(group_sizes && offsets && (T == 0 || (source_order && inverse)), "router: null pointer argument");
+  if (workspace_bytes < jtmoe_router_workspace_bytes(E))
+    return fail(JTMOE_EWORKSPACE, "router: workspace %zu < %zu bytes", workspace_bytes, jtmoe_router_workspace_bytes(E));
+  LayerPlan layer{group_sizes, offsets, source_order, inverse, false, false};
+  if (dtype == JTMOE_BF16)
+    rc = launch_router<bf16_raw, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
+                                        scores, expert_counts, importance, nullptr, workspace, s, &layer);
+  else
+    rc = launch_router<float, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
+                                     scores, expert_counts, importance, nullptr, workspace, s, &layer);
+  *stats_done = layer.stats_done;
+  *plan_done = layer.plan_done;
+  return rc;
+}
+
 }  // namespace jtmoe
 
 using namespace jtmoe;

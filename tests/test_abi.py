@@ -41,7 +41,7 @@ def test_workspace_sizing_is_pure_host_arithmetic():
     total = lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, _ffi.JTMOE_BF16)
     A = T * K
     payload = 2 * (A * H + A * I + A * H + T * Is + T * H)
-    assert payload <= total <= payload + 2**21  # + metadata, alignment and the router's partial sums (1 MiB at E=64)
+    assert payload <= total <= payload + 2**21  # + metadata, alignment and the router's partial sums (0.5 MiB at E=64)
     assert total % 256 == 0
     assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, _ffi.JTMOE_F32) >= 2 * payload
     assert lib.jtmoe_workspace_bytes(0, H, E, K, I, 0, _ffi.JTMOE_BF16) > 0

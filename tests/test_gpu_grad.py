@@ -331,6 +331,6 @@ def test_sequence_balance_loss_gradient_matches_oracle(gpu, batch, seq, experts,
     # through autograd, with a weight on the loss as the training objective applies it
     s_req = sd.clone().requires_grad_(True)
     loss = autograd.sequence_balance_loss(idd, s_req, top_k)
-    assert float(loss) == pytest.approx(float(O.sequence_balance_loss(ids, scores, top_k)), rel=1e-5)
+    assert float(loss.detach()) == pytest.approx(float(O.sequence_balance_loss(ids, scores, top_k)), rel=1e-5)
     (g,) = torch.autograd.grad(loss * 0.25, [s_req])
     np.testing.assert_allclose(host(g) / scale, 0.25 * want / scale, rtol=1e-4, atol=2e-6)

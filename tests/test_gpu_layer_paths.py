@@ -1,0 +1,85 @@
+"""The fused layer call and the stand-alone router + dispatch entry points give the same bits.
+
+Inside jtmoe_moe_forward the router leaves work to the dispatch behind it: at large batches the
+per-expert statistics (expert_counts / importance of _router_stats, moe.py:802-805) are summed by the
+dispatch's histogram pass instead of by the router's atomics, and at small batches the router's
+finishing workgroup writes the dispatch plan itself.  Whatever route a shape takes, every routing
+output of the layer must equal, bit for bit, what jtmoe_router followed by jtmoe_dispatch return on
+the same inputs (those two are tied to the oracle by test_gpu_parity.py); the statistics are sums in
+32.32 fixed point, so the order of summation cannot show.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from research_amd import ops
+from test_gpu_parity import dev, host
+
+pytestmark = pytest.mark.gpu
+
+# (tokens, hidden, experts, top_k, d_ff, dtype): the routes are chosen by tokens, tokens * top_k,
+# the dtype and whether hidden / experts suit the matrix-core router
+CASES = [
+    (0, 128, 16, 2, 64, "bf16"),      # empty batch: zeros everywhere
+    (5, 128, 16, 2, 64, "bf16"),      # finishing workgroup writes the plan
+    (64, 2048, 64, 8, 128, "bf16"),   # the decode shape of the benchmark
+    (200, 256, 256, 16, 64, "bf16"),  # 256 experts: the 64-token finishing workgroup is out, tokens > 64
+    (50, 256, 256, 16, 64, "bf16"),   # 256 experts: 64-token finishing workgroup with the plan
+    (256, 128, 32, 8, 64, "bf16"),    # the largest batch of the small-batch router
+    (257, 128, 32, 8, 64, "bf16"),    # 64-token workgroups, one-workgroup dispatch with the statistics
+    (1024, 128, 128, 8, 64, "bf16"),  # 8192 assignments: the largest one-workgroup dispatch
+    (1025, 128, 128, 8, 64, "bf16"),  # 8200 assignments: histogram and rank passes with the statistics
+    (5000, 192, 64, 6, 64, "bf16"),   # several chunks, ragged last chunk: histogram + rank passes
+    (33000, 128, 48, 8, 64, "bf16"),  # 258 chunks: histogram, scan and rank passes
+    (300, 100, 24, 3, 40, "bf16"),    # hidden and experts the matrix-core router does not take
+    (7, 48, 5, 2, 24, "f32"),
+    (2100, 64, 8, 4, 32, "f32"),      # fp32: generic router, 8400 assignments
+    (0, 64, 8, 4, 32, "f32"),
+]
+
+
+@pytest.mark.parametrize("tokens,hidden,experts,top_k,d_ff,dtype", CASES)
+def test_layer_routing_outputs_equal_the_stand_alone_entry_points(gpu, tokens, hidden, experts, top_k, d_ff, dtype):
+    rng = np.random.default_rng(tokens * 31 + experts)
+    x = dev(rng.standard_normal((tokens, hidden)).astype(np.float32), gpu, dtype)
+    w_router = dev((rng.standard_normal((hidden, experts)) * 0.1).astype(np.float32), gpu, dtype)
+    bias = dev((rng.standard_normal(experts) * 0.01).astype(np.float32), gpu)
+    gate = dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, dtype)
+    up = dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, dtype)
+    down = dev((rng.standard_normal((experts, d_ff, hidden)) * 0.05).astype(np.float32), gpu, dtype)
+
+    layer = ops.moe_forward(x, w_router, bias, gate, up, down, top_k, 1.5)
+    route = ops.router(x, w_router, bias, top_k, 1.5)
+    plan = ops.dispatch(route.expert_ids, experts)
+
+    for name in ("expert_ids", "weights", "scores", "expert_counts", "importance"):
+        assert torch.equal(getattr(layer, name), getattr(route, name)), name
+    for name in ("group_sizes", "offsets", "source_order", "inverse"):
+        assert torch.equal(getattr(layer, name), getattr(plan, name)), name
+    # and the statistics are what the ids and weights say
+    stats = O.router_stats(host(route.expert_ids), host(route.weights), experts)
+    assert np.array_equal(host(layer.expert_counts), stats.expert_counts)
+    np.testing.assert_allclose(host(layer.importance), stats.importance, rtol=1e-5, atol=1e-5)
+    assert int(layer.group_sizes.sum()) == tokens * top_k
+
+
+def test_layer_statistics_do_not_depend_on_what_the_buffers_held(gpu):
+    """The layer's scratch is never cleared between calls: a second call on other inputs through the same
+    workspace and output buffers must not see the first one's sums."""
+    rng = np.random.default_rng(9)
+    H, E, K, I = 128, 32, 4, 64
+    w_router = dev((rng.standard_normal((H, E)) * 0.1).astype(np.float32), gpu, "bf16")
+    gate = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    up = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    down = dev((rng.standard_normal((E, I, H)) * 0.05).astype(np.float32), gpu, "bf16")
+    for tokens in (4096, 3000, 40, 4096):
+        x = dev(rng.standard_normal((tokens, H)).astype(np.float32), gpu, "bf16")
+        layer = ops.moe_forward(x, w_router, None, gate, up, down, K, 1.0)
+        route = ops.router(x, w_router, None, K, 1.0)
+        assert torch.equal(layer.expert_counts, route.expert_counts), tokens
+        assert torch.equal(layer.importance, route.importance), tokens
+        assert float(layer.expert_counts.sum()) == tokens * K

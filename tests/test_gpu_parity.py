@@ -157,7 +157,10 @@ def check_dispatch(gpu, ids: np.ndarray, experts: int, x: np.ndarray | None, dty
     [(1, 1, 1, 8, "f32"), (6, 2, 4, 3, "f32"), (511, 2, 8, 64, "bf16"), (512, 2, 8, 64, "bf16"), (513, 2, 8, 64, "bf16"),
      (1000, 8, 64, 256, "bf16"), (4096, 8, 128, 40, "bf16"), (333, 3, 256, 7, "bf16"), (2048, 2, 16, 1024, "f32"),
      # either side of the single-workgroup limit (8192 assignments)
-     (1024, 8, 32, 8, "bf16"), (8193, 1, 32, 8, "bf16"), (700, 4, 256, 8, "bf16")],
+     (1024, 8, 32, 8, "bf16"), (8193, 1, 32, 8, "bf16"), (700, 4, 256, 8, "bf16"),
+     # either side of the chunk count (256 chunks of 1024 assignments) up to which the rank pass does the
+     # scan itself, and a batch far beyond it with an odd expert count
+     (32768, 8, 64, 8, "bf16"), (262145, 1, 24, 8, "bf16"), (150001, 4, 255, 8, "bf16")],
 )
 def test_dispatch_is_bit_exact(gpu, tokens, top_k, experts, hidden, dtype):
     rng = np.random.default_rng(tokens + experts)
