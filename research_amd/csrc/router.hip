@@ -128,47 +128,54 @@ __device__ __forceinline__ float quad_xor_f32(float v) {
   return __builtin_bit_cast(float, quad_xor_i32<kXor>(__builtin_bit_cast(int, v)));
 }
 
+// Order-preserving map of a non-NaN float onto a signed integer: a > b as floats <=> key(a) > key(b)
+// (-0 is canonicalised to +0 first, so equal floats have equal keys).  No float maps to INT_MIN,
+// which therefore serves as "already taken".
+__device__ __forceinline__ int order_key(float v) {
+  const int bits = __builtin_bit_cast(int, v + 0.0f);
+  return bits ^ ((bits >> 31) & 0x7fffffff);
+}
+constexpr int kTakenKey = (int)0x80000000u;
+
 // K rounds of "largest remaining score + bias, lower index on ties" for one token, by its four
-// lanes: lane q owns experts [e_begin, e_begin + EQ) and keeps them in registers.
+// lanes: lane q owns experts [e_begin, e_begin + EQ) and keeps their keys in registers; a taken
+// expert's key becomes kTakenKey, below every real value, so a round is one compare and two
+// selects per expert.
 template <int EQ>
 __device__ __forceinline__ void select_from_registers(const RouterSmem& sm, const float* row, int e_begin, bool row_ok,
                                                       int t, int q, int K) {
 #pragma clang fp contract(off)
-  float v[EQ];
+  int key[EQ];
 #pragma unroll
-  for (int j = 0; j < EQ; ++j) v[j] = row_ok ? row[e_begin + j] + sm.bias[e_begin + j] : 0.0f;
-  unsigned long long taken = 0ull;
+  for (int j = 0; j < EQ; ++j) key[j] = row_ok ? order_key(row[e_begin + j] + sm.bias[e_begin + j]) : kTakenKey;
   for (int r = 0; r < K; ++r) {
-    float best_v = 0.0f;
-    int best_e = -1;
-    if (row_ok) {
+    int best_k = kTakenKey, best_e = -1;
 #pragma unroll
-      for (int j = 0; j < EQ; ++j) {
-        if (!((taken >> j) & 1ull) && (best_e < 0 || v[j] > best_v)) {
-          best_v = v[j];
-          best_e = e_begin + j;
-        }
-      }
+    for (int j = 0; j < EQ; ++j) {
+      const bool better = key[j] > best_k;  // strictly: the lower index keeps a tie
+      best_k = better ? key[j] : best_k;
+      best_e = better ? e_begin + j : best_e;
     }
     {
-      const float ov = quad_xor_f32<1>(best_v);
+      const int ok = quad_xor_i32<1>(best_k);
       const int oe = quad_xor_i32<1>(best_e);
-      if (oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e))) {
-        best_v = ov;
+      if (oe >= 0 && (best_e < 0 || ok > best_k || (ok == best_k && oe < best_e))) {
+        best_k = ok;
         best_e = oe;
       }
     }
     {
-      const float ov = quad_xor_f32<2>(best_v);
+      const int ok = quad_xor_i32<2>(best_k);
       const int oe = quad_xor_i32<2>(best_e);
-      if (oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e))) {
-        best_v = ov;
+      if (oe >= 0 && (best_e < 0 || ok > best_k || (ok == best_k && oe < best_e))) {
+        best_k = ok;
         best_e = oe;
       }
     }
     if (row_ok) {
-      const int j = best_e - e_begin;
-      if (j >= 0 && j < EQ) taken |= 1ull << j;
+      const int own = best_e - e_begin;
+#pragma unroll
+      for (int j = 0; j < EQ; ++j) key[j] = j == own ? kTakenKey : key[j];
       if (q == 0) {
         sm.top_id[t * K + r] = best_e;
         sm.top_score[t * K + r] = row[best_e];
