@@ -73,6 +73,7 @@ struct Problem {
 
 // rows are spread over E groups (skewed, some empty); with top_k > 0 the A matrix has
 // rows/top_k rows and packed row j reads A row row_map[j] / top_k (gather on load)
+static bool g_equal_groups = false;  // every group rows / E rows (no ragged last tiles) instead of random sizes
 static Problem make(int E, int rows, int K, int N, unsigned seed, bool skew, int top_k, float scale) {
   Problem p;
   p.E = E; p.rows = rows; p.K = K; p.N = N; p.top_k = top_k;
@@ -81,6 +82,7 @@ static Problem make(int E, int rows, int K, int N, unsigned seed, bool skew, int
   for (int r = 0; r < rows; ++r) {
     int e = skew ? (int)(std::pow((double)(rng() % 10000) / 10000.0, 3.0) * E) : (int)(rng() % E);
     if (skew && e % 5 == 3) e = 0;
+    if (g_equal_groups) e = r % E;
     p.gs[e]++;
   }
   p.off.assign(E, 0);
@@ -652,6 +654,26 @@ int main(int argc, char** argv) {
       g_stream = false;
     }
     release(sq);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_ragged")) {
+    // What the ragged last tile of every group costs: the C3 launches on groups of random sizes
+    // (about 2048 +- 45 rows: 544 row tiles, 64 of them partly filled) and on 64 groups of exactly
+    // 2048 rows (512 full row tiles).
+    Problem g = make(64, 131072, 2048, 1408, 4, false, 8, 1.0f);
+    Problem d = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
+    g_equal_groups = true;
+    Problem ge = make(64, 131072, 2048, 1408, 4, false, 8, 1.0f);
+    Problem de = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
+    g_equal_groups = false;
+    for (int rep = 0; rep < 3; ++rep) {
+      g_stream = true;
+      timeit<GateUpStreamCfg>("gate/up stream, random group sizes", g, 20);
+      timeit<GateUpStreamCfg>("gate/up stream, equal groups", ge, 20);
+      g_stream = false;
+      timeit<DownCfg>("down library, random group sizes", d, 20);
+      timeit<DownCfg>("down library, equal groups", de, 20);
+    }
+    release(g); release(d); release(ge); release(de);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_ablation")) {
     // What bounds the stream kernel: the same launch with parts of the k loop left out (results are

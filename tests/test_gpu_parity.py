@@ -80,6 +80,31 @@ def test_routing_decision_is_bit_exact_given_logits(gpu, tokens, experts, top_k,
     np.testing.assert_allclose(host(got.importance), stats.importance, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("experts,top_k", [(64, 8), (128, 8), (16, 4), (24, 3), (256, 16)])
+def test_routing_decision_with_negative_zero_and_infinite_biased_scores(gpu, experts, top_k):
+    """The selection compares score + bias.  Biases of either sign and any size make those sums
+    negative, exactly zero (both signs of zero compare equal) or infinite; the order must stay
+    "value descending, lower index on ties" through all of them (expert counts with and without the
+    register-resident selection)."""
+    rng = np.random.default_rng(experts)
+    tokens = 400
+    logits = O.bf16_round((rng.standard_normal((tokens, experts)) * 2.0).astype(np.float32))
+    logits[0, :] = 0.0
+    bias = (rng.standard_normal(experts) * 2.0).astype(np.float32)  # most sums negative for half the experts
+    bias[1] = -np.inf   # never selected while K finite candidates remain
+    bias[2] = np.inf    # always first
+    bias[3] = -0.0
+    bias[4] = -0.5      # row 0: score 0.5 + bias = +0.0 exactly, tied with nothing else by value
+    bias[5] = -0.5      # ... and tied with expert 4: the lower index wins
+    bias[6] = -np.inf
+    want = O.router_from_logits(logits, bias, top_k, 1.0, "bf16")
+    got = ops.router_from_logits(dev(logits, gpu), dev(bias, gpu), top_k, 1.0, dtype=torch.bfloat16)
+    assert np.array_equal(host(got.expert_ids), want.expert_ids)
+    assert np.array_equal(host(got.weights), want.weights)
+    assert np.all(host(got.expert_ids)[:, 0] == 2)
+    assert not np.any(np.isin(host(got.expert_ids), [1, 6]))
+
+
 @pytest.mark.parametrize("case", ["router_order", "router_bias_scale"])
 def test_router_known_answers(gpu, kat, case):
     c = kat[case]
