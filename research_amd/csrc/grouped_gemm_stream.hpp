@@ -61,19 +61,27 @@ struct StreamLayout {
   static_assert(Cfg::BM <= Cfg::NT, "one row-map entry per thread");
 };
 
-template <typename Cfg>
-__global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
-    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
-    uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
-    int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
-    int a_rows, uint16_t* __restrict__ save0, uint16_t* __restrict__ save1, int window, int chunk) {
+// kNT = false: C = A @ B[e] with B[e] stored [K, N] (the forward products; kDual: two of them sharing the A tile).
+// kNT = true:  C = sum over segs segments of A_s @ B_s[e]^T with B_s[e] stored [N, K] (the data gradients of
+//              the backward pass, grouped_gemm_bwd.hpp): the B tile is then k-contiguous like the A tile,
+//              lives in LDS in the same swizzled row layout and is read with ds_read_b128; the k loop
+//              runs through the segments one after the other.
+template <typename Cfg, bool kNT>
+__device__ __forceinline__ void stream_gemm_body(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ A1, const uint16_t* __restrict__ B0,
+    const uint16_t* __restrict__ B1, uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes,
+    const int32_t* __restrict__ offsets, int E, int dense_rows, int Kdim, int N, int mtiles, int ntiles_n,
+    const int32_t* __restrict__ row_map, int row_div, int a_rows, uint16_t* __restrict__ save0,
+    uint16_t* __restrict__ save1, int segs, int window, int chunk) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, NS = Cfg::NSTAGE;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   constexpr int CPRA = Cfg::CPRA, KK = BK / 16, LPS = Cfg::LPS;
   constexpr bool kDual = Cfg::kDual;
   using L = StreamLayout<Cfg>;
   static_assert(KK % 2 == 0, "fragment double buffer wants an even number of sub-steps");
-  static_assert((Cfg::OPT & 128) != 0, "weight tiles in 4 x 64 blocks");
+  static_assert(kNT || (Cfg::OPT & 128) != 0, "weight tiles in 4 x 64 blocks");
+  static_assert(!kNT || !kDual, "the transposed-B form has one output per tile");
+  static_assert(!kNT || (BN * CPRA) % NT == 0, "the B tile must divide evenly over the threads");
   // Timing experiments of the stand-alone check (wrong results by construction, never launched by the
   // library): OPT & 256 leaves out the operand loads of the steady part of the k loop, OPT & 512 its
   // fragment reads (the MFMAs then run on the fragments read once before the loop).
@@ -87,7 +95,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WAVES_N, wn = wave - wm * Cfg::WAVES_N;
   const bool gather = row_map != nullptr;
-  const int nk = Kdim / BK;
+  const int nk1 = Kdim / BK;               // k steps of one segment
+  const int nk = kNT ? nk1 * segs : nk1;   // k steps of a tile
 
   // ---- schedule (as in grouped_gemm_dma_persistent_kernel) ----
   // Group sizes and first rows are copied into LDS once; every tile look-up scans them from there, so
@@ -143,11 +152,15 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   // ---- the load plan: descriptors and offsets of the tile whose operands are being requested.  The
   // last NS steps of a tile request the next tile's first steps, so the plan switches over to the next
   // tile NS steps before the current tile ends; nothing else of the current tile depends on it. ----
+  constexpr int NSEG = kNT ? 2 : 1;                        // A descriptors (one per segment)
+  constexpr int NBD = kNT ? 2 : Cfg::NSUB;                 // B descriptors (per segment / per 128-column sub-tile)
+  constexpr int B_LOADS = kNT ? BN * CPRA / NT : Cfg::NSUB;  // entries of b_voff
+  static_assert(!kNT || B_LOADS == Cfg::NSUB * Cfg::BSUB_LOADS, "a stage has LPS loads in either form");
   struct Plan {
-    i32x4_t a_rsrc;
-    i32x4_t b_rsrc[Cfg::NSUB];
+    i32x4_t a_rsrc[NSEG];
+    i32x4_t b_rsrc[NBD];
     int a_voff[Cfg::A_LOADS];
-    int b_voff[Cfg::NSUB];
+    int b_voff[B_LOADS];
   };
   const int a_r = tid / CPRA, a_slot = tid - a_r * CPRA;
   const int a_c = a_slot ^ ((a_r / (16 / CPRA)) % CPRA);
@@ -161,11 +174,24 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   // everything of a plan but the A row offsets
   auto plan_tile = [&](Plan& p, const Tile& t) {
     const size_t wofs = (size_t)t.expert * Kdim * N;
+    if constexpr (kNT) {
 #pragma unroll
-    for (int u = 0; u < Cfg::NSUB; ++u) p.b_rsrc[u] = make_rsrc((kDual && u == 1 ? B1 : B0) + wofs, Kdim * N * 2);
-    p.a_rsrc = gather ? make_rsrc(A, a_rows * Kdim * 2) : make_rsrc(A + (size_t)t.row0 * Kdim, t.rows * Kdim * 2);
+      for (int sg = 0; sg < 2; ++sg) {
+        const uint16_t* a = (sg == 1 && segs > 1) ? A1 : A;
+        const uint16_t* b = (sg == 1 && segs > 1) ? B1 : B0;
+        p.a_rsrc[sg] = gather ? make_rsrc(a, a_rows * Kdim * 2) : make_rsrc(a + (size_t)t.row0 * Kdim, t.rows * Kdim * 2);
+        p.b_rsrc[sg] = make_rsrc(b + wofs, N * Kdim * 2);  // rows of B past N lie outside it and read as zeros
+      }
+      // the B tile's rows are output columns: row n0 + r of B[e], the same slots and swizzle as the A tile
 #pragma unroll
-    for (int u = 0; u < Cfg::NSUB; ++u) p.b_voff[u] = (b_k * N + t.n0 + (kDual ? 0 : u * 128) + b_c * 8) * 2;
+      for (int j = 0; j < B_LOADS; ++j) p.b_voff[j] = ((t.n0 + a_r + j * (NT / CPRA)) * Kdim + a_c * 8) * 2;
+    } else {
+#pragma unroll
+      for (int u = 0; u < Cfg::NSUB; ++u) p.b_rsrc[u] = make_rsrc((kDual && u == 1 ? B1 : B0) + wofs, Kdim * N * 2);
+      p.a_rsrc[0] = gather ? make_rsrc(A, a_rows * Kdim * 2) : make_rsrc(A + (size_t)t.row0 * Kdim, t.rows * Kdim * 2);
+#pragma unroll
+      for (int u = 0; u < Cfg::NSUB; ++u) p.b_voff[u] = (b_k * N + t.n0 + (kDual ? 0 : u * 128) + b_c * 8) * 2;
+    }
 #pragma unroll
     for (int j = 0; j < Cfg::A_LOADS; ++j) p.a_voff[j] = ((a_r + j * (NT / CPRA)) * Kdim + a_c * 8) * 2;
   };
@@ -182,30 +208,31 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
       p.a_voff[j] = r < t.rows ? (src * Kdim + a_c * 8) * 2 : 0x70000000;
     }
   };
-  auto issue = [&](const Plan& p, int kt, int stage) {
-    const unsigned base = wave_lds + stage * Cfg::STAGE_BYTES;
-    const int k0 = kt * BK;
-#pragma unroll
-    for (int j = 0; j < Cfg::A_LOADS; ++j) buffer_load_lds16(p.a_rsrc, base + j * NT * 16, p.a_voff[j], k0 * 2);
-#pragma unroll
-    for (int u = 0; u < Cfg::NSUB; ++u)
-#pragma unroll
-      for (int j = 0; j < Cfg::BSUB_LOADS; ++j)
-        buffer_load_lds16(p.b_rsrc[u], base + Cfg::A_BYTES + u * Cfg::BSUB_BYTES + j * NT * 16,
-                          p.b_voff[u] + j * (NT / 16) * N * 2, k0 * N * 2);
-  };
-
-  // load i of the LPS loads of a stage (A loads first, then the B sub-tiles)
+  // load i of the LPS loads of a stage (A loads first, then B) of k step kt of the planned tile
   auto issue_one = [&](const Plan& p, int kt, int stage, int i) {
     const unsigned base = wave_lds + stage * Cfg::STAGE_BYTES;
-    const int k0 = kt * BK;
-    if (i < Cfg::A_LOADS) {
-      buffer_load_lds16(p.a_rsrc, base + i * NT * 16, p.a_voff[i], k0 * 2);
+    if constexpr (kNT) {
+      const bool second = kt >= nk1;  // uniform: the step belongs to the second segment
+      const int k0 = (second ? kt - nk1 : kt) * BK;
+      if (i < Cfg::A_LOADS)
+        buffer_load_lds16(second ? p.a_rsrc[1] : p.a_rsrc[0], base + i * NT * 16, p.a_voff[i], k0 * 2);
+      else
+        buffer_load_lds16(second ? p.b_rsrc[1] : p.b_rsrc[0], base + Cfg::A_BYTES + (i - Cfg::A_LOADS) * NT * 16,
+                          p.b_voff[i - Cfg::A_LOADS], k0 * 2);
     } else {
-      const int u = (i - Cfg::A_LOADS) / Cfg::BSUB_LOADS, jb = (i - Cfg::A_LOADS) % Cfg::BSUB_LOADS;
-      buffer_load_lds16(p.b_rsrc[u], base + Cfg::A_BYTES + u * Cfg::BSUB_BYTES + jb * NT * 16,
-                        p.b_voff[u] + jb * (NT / 16) * N * 2, k0 * N * 2);
+      const int k0 = kt * BK;
+      if (i < Cfg::A_LOADS) {
+        buffer_load_lds16(p.a_rsrc[0], base + i * NT * 16, p.a_voff[i], k0 * 2);
+      } else {
+        const int u = (i - Cfg::A_LOADS) / Cfg::BSUB_LOADS, jb = (i - Cfg::A_LOADS) % Cfg::BSUB_LOADS;
+        buffer_load_lds16(p.b_rsrc[u], base + Cfg::A_BYTES + u * Cfg::BSUB_BYTES + jb * NT * 16,
+                          p.b_voff[u] + jb * (NT / 16) * N * 2, k0 * N * 2);
+      }
     }
+  };
+  auto issue = [&](const Plan& p, int kt, int stage) {
+#pragma unroll
+    for (int i = 0; i < LPS; ++i) issue_one(p, kt, stage, i);
   };
 
   // ---- fragment addresses of this lane (bytes inside a stage) ----
@@ -215,6 +242,10 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   const int b_laneoff = ((lane & 15) >> 2) * 128 + (lane & 3) * 8 + ((lane >> 4) & 1) * 32 + (lane >> 5) * 2048;
   const int half_swap = ((lane >> 3) & 1) * 64;
   int b_blk[TN];
+  // kNT: the B tile in the A tile's layout, this lane's row = its output column
+  const int bt_row = wn * WN + (lane & 31);
+  const int bt_sw = (bt_row / (16 / CPRA)) % CPRA;
+  const int bt_rowoff = Cfg::A_BYTES + bt_row * (BK * 2);
 #pragma unroll
   for (int jj = 0; jj < TN; ++jj) {
     int col;
@@ -231,6 +262,10 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
     return *reinterpret_cast<const bf16x8_t*>(st + a_rowoff + mi * 32 * BK * 2 + (((kk * 2 + (lane >> 5)) ^ a_sw) << 4));
   };
   auto load_frag_b = [&](int stage, int kk, int jj) -> bf16x8_t {
+    if constexpr (kNT) {
+      const unsigned char* st = smem_raw + stage * Cfg::STAGE_BYTES;
+      return *reinterpret_cast<const bf16x8_t*>(st + bt_rowoff + jj * 32 * BK * 2 + (((kk * 2 + (lane >> 5)) ^ bt_sw) << 4));
+    }
     const unsigned char* p = smem_raw + stage * Cfg::STAGE_BYTES + b_blk[jj] + b_laneoff + kk * (4 * 8 * 128);
     const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
     const s16x4_t hi =
@@ -459,6 +494,28 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
   }
 }
 
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_kernel(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
+    uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
+    int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
+    int a_rows, uint16_t* __restrict__ save0, uint16_t* __restrict__ save1, int window, int chunk) {
+  stream_gemm_body<Cfg, false>(A, nullptr, B0, B1, C, group_sizes, offsets, E, dense_rows, Kdim, N, mtiles, ntiles_n,
+                               row_map, row_div, a_rows, save0, save1, 1, window, chunk);
+}
+
+// The transposed-B form: the arguments of grouped_gemm_nt_kernel (grouped_gemm_bwd.hpp) plus the schedule.
+// Requirements: (Kdim / BK) * segs >= 2 * NSTAGE, and those of the kernel above.
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_nt_kernel(
+    const uint16_t* __restrict__ A0, const uint16_t* __restrict__ A1, const uint16_t* __restrict__ B0,
+    const uint16_t* __restrict__ B1, uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes,
+    const int32_t* __restrict__ offsets, int E, int dense_rows, int Kdim, int N, int mtiles, int ntiles_n,
+    const int32_t* __restrict__ row_map, int row_div, int a_rows, int segs, int window, int chunk) {
+  stream_gemm_body<Cfg, true>(A0, A1, B0, B1, C, group_sizes, offsets, E, dense_rows, Kdim, N, mtiles, ntiles_n,
+                              row_map, row_div, a_rows, nullptr, nullptr, segs, window, chunk);
+}
+
 // The configuration the library launches for gate/up (routed and shared experts): the tile of GateUpCfg
 // with 32-deep steps and four stages.  Measured on 64 groups of 2048 gathered rows x 2048 x 1408
 // (alternating in one process): 1.306 ms against 1.400-1.409 ms for grouped_gemm_dma_persistent_kernel
@@ -470,5 +527,7 @@ using GateUpStreamCfg = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128>;
 using GateUpStream2Cfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
 using DownStreamCfg = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768>;
 using DownStream2Cfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 128 + 32768>;
+// The data-gradient products of the backward pass (transposed-B form): 256 x 256 tiles, 2 x 4 waves.
+using DgradStreamCfg = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128>;
 
 }  // namespace jtmoe

@@ -7,6 +7,11 @@
 //   gemm_check time_backward   + timing of the four backward launches at the C3 shape
 //   gemm_check time       + timing of the library's two configurations at the C3 shape,
 //                           once on N(0,1)-like data and once on all-zero data
+//   gemm_check time_stream / time_ablation / counters_stream   the stream kernel against the older one,
+//                           with parts of its loop left out, and a fixed launch sequence for counter runs
+//   gemm_check time_stream_nt   the transposed-B form of the stream kernel against grouped_gemm_nt_kernel
+//   gemm_check time_ragged      the C3 launches on random against equal group sizes
+//   (a second argument "nocheck" skips the correctness cases)
 #include "grouped_gemm_bwd.hpp"
 #include "grouped_gemm_stream.hpp"
 
@@ -285,8 +290,39 @@ static bool compare(const char* name, const float* dref, const uint16_t* dgot, s
   return bad == 0;
 }
 
+// the transposed-B form of the stream kernel (what the library launches for the data gradients where it fits)
+static int g_stream_nt = 0;  // 0: the older kernel; 1: DgradStreamCfg; 2 and 3: its variants below
+using DgradStream42Cfg = DmaGemmCfg<256, 256, 32, 4, 2, false, 4, 16 + 128>;  // 4 x 2 waves of 64 x 128
+using DgradStream2Cfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 128>;   // 64-deep steps, two stages
+template <typename Cfg>
+static void launch_stream_nt_cfg(Problem& p, const uint16_t* A1, int segs, bool dense) {
+  using L = StreamLayout<Cfg>;
+  if ((p.K / Cfg::BK) * segs < 2 * Cfg::NSTAGE || p.K % Cfg::BK != 0) {
+    printf("stream nt: K=%d segs=%d is outside the kernel's envelope\n", p.K, segs);
+    exit(1);
+  }
+  auto kernel = grouped_gemm_stream_nt_kernel<Cfg>;
+  CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                         (int)L::kSmemBytes));
+  const long mt = dense ? (p.rows + Cfg::BM - 1) / Cfg::BM
+                        : (p.rows + Cfg::BM - 1) / Cfg::BM + (p.E < p.rows ? p.E : p.rows);
+  const long nt = (p.N + Cfg::BN - 1) / Cfg::BN;
+  const long tiles_grid = gemm_grid(mt, nt);
+  PersistentSchedule ps = persistent_schedule(tiles_grid, 256, g_chunk < 0 ? kTilesPerWorkgroup<Cfg> : g_chunk);
+  if (tiles_grid <= 256) ps = {tiles_grid, 0, 0};
+  kernel<<<(unsigned)ps.grid, Cfg::NT, L::kSmemBytes>>>(
+      p.A, A1, p.B0, p.B1, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows, p.K, p.N, (int)mt,
+      (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, segs, ps.window, ps.chunk);
+}
+static void launch_stream_nt(Problem& p, const uint16_t* A1, int segs, bool dense) {
+  if (g_stream_nt == 2) return launch_stream_nt_cfg<DgradStream42Cfg>(p, A1, segs, dense);
+  if (g_stream_nt == 3) return launch_stream_nt_cfg<DgradStream2Cfg>(p, A1, segs, dense);
+  launch_stream_nt_cfg<DgradStreamCfg>(p, A1, segs, dense);
+}
+
 template <typename Cfg>
 static void launch_nt(Problem& p, const uint16_t* A1, int segs, bool dense) {
+  if (g_stream_nt) return launch_stream_nt(p, A1, segs, dense);
   auto kernel = grouped_gemm_nt_kernel<Cfg>;
   CK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                          (int)Cfg::SMEM_BYTES));
@@ -390,7 +426,7 @@ static void time_launches(const char* name, double flops, int iters, F launch_on
   float ms;
   CK(hipEventElapsedTime(&ms, a, b));
   ms /= iters;
-  printf("time %-44s %.3f ms  %.1f TFLOP/s  (%.1f%% of 2500)\n", name, ms, flops / ms / 1e9, flops / ms / 1e9 / 25.0);
+  printf("time %-52s %.3f ms  %.1f TFLOP/s  (%.1f%% of 2500)\n", name, ms, flops / ms / 1e9, flops / ms / 1e9 / 25.0);
   fflush(stdout);
 }
 
@@ -622,6 +658,27 @@ int main(int argc, char** argv) {
     g_chunk = -1;
     release(v);
     g_stream = false;
+    // the transposed-B form of the stream kernel
+    for (g_stream_nt = 1; g_stream_nt <= 3; ++g_stream_nt) {
+    Problem w1 = make(7, 3001, 576, 392, 61, true, 0, 1.0f);  // ragged groups, N not a multiple of the tile
+    ok &= check_nt<DgradCfg>("stream dgrad ragged", w1, 1);
+    ok &= check_nt<DgradCfg>("stream dgrad ragged, two segments", w1, 2);
+    release(w1);
+    Problem w2 = make(5, 2400, 512, 384, 62, true, 3, 1.0f);
+    ok &= check_nt<DgradCfg>("stream dgrad gather on load", w2, 1);
+    release(w2);
+    Problem w3 = make(1, 777, 512, 520, 63, false, 0, 1.0f);
+    ok &= check_nt<DgradCfg>("stream dgrad dense, two segments", w3, 2, true);
+    release(w3);
+    Problem w4 = make(40, 70000, 256, 264, 64, true, 0, 1.0f);  // many more tiles than workgroups
+    ok &= check_nt<DgradCfg>("stream dgrad many tiles per workgroup", w4, 1);
+    ok &= check_nt<DgradCfg>("stream dgrad many tiles per workgroup, two segments", w4, 2);
+    release(w4);
+    Problem w5 = make(33, 90000, 128, 392, 65, true, 4, 1.0f);  // 4 k steps per segment: two segments just fill the pipeline
+    ok &= check_nt<DgradCfg>("stream dgrad short segments, gather", w5, 2);
+    release(w5);
+    }
+    g_stream_nt = 0;
   }
   }  // !nocheck
   if (ok && argc > 1 && !strcmp(argv[1], "time_stream")) {
@@ -654,6 +711,26 @@ int main(int argc, char** argv) {
       g_stream = false;
     }
     release(sq);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_stream_nt")) {
+    // the data-gradient products of the C3 backward pass: older kernel against the stream form
+    const int rows = 131072, H = 2048, I = 1408, E = 64;
+    Problem z = make(E, rows, H, I, 21, false, 0, 1.0f);   // Z = dYp @ Wd^T : A [rows, H], B [E, I, H]
+    Problem x = make(E, rows, I, H, 22, false, 0, 1.0f);   // dXp = dG @ Wg^T + dU @ Wu^T : A [rows, I] twice, B [E, H, I] twice
+    uint16_t* A1 = random_bf16((size_t)rows * I, 33, 1.0f);
+    for (int rep = 0; rep < 3; ++rep) {
+      const char* names[4] = {"older kernel", "stream 4 x 32, 2 x 4 waves", "stream 4 x 32, 4 x 2 waves", "stream 2 x 64, 2 x 4 waves"};
+      for (g_stream_nt = 0; g_stream_nt <= 3; ++g_stream_nt) {
+        char label[96];
+        snprintf(label, sizeof label, "Z = dYp @ Wd^T, %s", names[g_stream_nt]);
+        time_launches(label, 2.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(z, nullptr, 1, false); });
+        snprintf(label, sizeof label, "dXp (2 segments), %s", names[g_stream_nt]);
+        time_launches(label, 4.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(x, A1, 2, false); });
+      }
+      g_stream_nt = 0;
+    }
+    hipFree(A1);
+    release(z); release(x);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_ragged")) {
     // What the ragged last tile of every group costs: the C3 launches on groups of random sizes
