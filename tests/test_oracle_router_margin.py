@@ -6,7 +6,7 @@ correctly-working logistic routines agree to within a few units in the last plac
 a different-but-valid routine could pick a different expert are those whose margin between the K-th
 and the (K+1)-th largest ``score + bias`` is at most a few fp32 ulp.  This test measures that
 fraction on the seed-0 inputs of the headline configuration (C3, bf16 logits) and on C1 (fp32
-logits), and prints it; DESIGN.md quotes the numbers.
+logits), prints it and asserts the figures that the design notes quote.
 
 Exact ties (margin 0) are not exposure: equal bf16 logits give equal scores under any deterministic
 sigmoid, and ties break towards the lower index in every implementation of the contract
