@@ -43,6 +43,19 @@ enum {
   JTMOE_ELAUNCH = -4       /* hipGetLastError() after a launch reported an error */
 };
 
+/*
+ * Score function of the router.  JTMOE_SCORE_SIGMOID is the reference's (moe.py:133) and what every
+ * entry point without the _sf suffix computes.  JTMOE_SCORE_SOFTMAX has no counterpart in the
+ * reference: the benchmark's second configuration names a softmax router, so it is offered as an
+ * attribute of the same router: scores = softmax over the experts of the fp32 logits, everything
+ * after the scores (biased top-k, renormalised weights, statistics) unchanged.  The _sf entry points
+ * take it right after route_scale and are otherwise their namesakes.
+ */
+enum {
+  JTMOE_SCORE_SIGMOID = 0,
+  JTMOE_SCORE_SOFTMAX = 1
+};
+
 /* Limits of the implementation. */
 #define JTMOE_MAX_EXPERTS 256
 #define JTMOE_MAX_TOP_K 16
@@ -72,6 +85,12 @@ int jtmoe_router(const void* x, const void* w_router, const float* expert_bias,
                  float* expert_counts, float* importance, float* logits,
                  void* workspace, size_t workspace_bytes, void* stream);
 
+int jtmoe_router_sf(const void* x, const void* w_router, const float* expert_bias,
+                    int64_t T, int64_t H, int64_t E, int64_t K, double route_scale, int score_func, int dtype,
+                    int32_t* expert_ids, void* weights, float* scores,
+                    float* expert_counts, float* importance, float* logits,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
 /*
  * The same router, starting from given fp32 logits [T,E] (moe.py:133-147 only).
  * The routing decision is a pure function of the logits, identical bit for bit
@@ -82,6 +101,11 @@ int jtmoe_router_from_logits(const float* logits, const float* expert_bias,
                              int32_t* expert_ids, void* weights, float* scores,
                              float* expert_counts, float* importance,
                              void* workspace, size_t workspace_bytes, void* stream);
+int jtmoe_router_from_logits_sf(const float* logits, const float* expert_bias,
+                                int64_t T, int64_t E, int64_t K, double route_scale, int score_func, int dtype,
+                                int32_t* expert_ids, void* weights, float* scores,
+                                float* expert_counts, float* importance,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Token dispatch.  Replaces the single-device part of local_dispatch
@@ -249,6 +273,16 @@ int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_b
                       int32_t* group_sizes, int32_t* offsets,
                       int32_t* source_order, int32_t* inverse,
                       void* workspace, size_t workspace_bytes, void* stream);
+int jtmoe_moe_forward_sf(const void* x, const void* w_router, const float* expert_bias,
+                         const void* gate, const void* up, const void* down,
+                         const void* shared_gate, const void* shared_up, const void* shared_down,
+                         int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                         double route_scale, int score_func, int dtype,
+                         void* y, int32_t* expert_ids, void* weights, float* scores,
+                         float* expert_counts, float* importance,
+                         int32_t* group_sizes, int32_t* offsets,
+                         int32_t* source_order, int32_t* inverse,
+                         void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Measurement aid with no counterpart in the reference (its benchmarks time
@@ -389,6 +423,12 @@ int jtmoe_router_backward(const void* x, const void* w_router,
                           int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
                           void* dx, void* d_w_router,
                           void* workspace, size_t workspace_bytes, void* stream);
+int jtmoe_router_backward_sf(const void* x, const void* w_router,
+                             const float* scores, const int32_t* expert_ids,
+                             const void* d_weights, const float* d_scores, double route_scale, int score_func,
+                             int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
+                             void* dx, void* d_w_router,
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The layer: jtmoe_moe_forward that also stores the residuals, and the VJP of
@@ -406,6 +446,17 @@ int jtmoe_moe_forward_train(const void* x, const void* w_router, const float* ex
                             int32_t* source_order, int32_t* inverse,
                             void* gate_pre, void* up_pre, void* shared_gate_pre, void* shared_up_pre,
                             void* workspace, size_t workspace_bytes, void* stream);
+int jtmoe_moe_forward_train_sf(const void* x, const void* w_router, const float* expert_bias,
+                               const void* gate, const void* up, const void* down,
+                               const void* shared_gate, const void* shared_up, const void* shared_down,
+                               int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                               double route_scale, int score_func, int dtype,
+                               void* y, int32_t* expert_ids, void* weights, float* scores,
+                               float* expert_counts, float* importance,
+                               int32_t* group_sizes, int32_t* offsets,
+                               int32_t* source_order, int32_t* inverse,
+                               void* gate_pre, void* up_pre, void* shared_gate_pre, void* shared_up_pre,
+                               void* workspace, size_t workspace_bytes, void* stream);
 
 size_t jtmoe_moe_backward_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
                                           int dtype);
@@ -422,6 +473,19 @@ int jtmoe_moe_backward(const void* x, const void* dy, const float* d_scores,
                        void* dx, void* d_w_router, void* d_gate, void* d_up, void* d_down,
                        void* d_shared_gate, void* d_shared_up, void* d_shared_down,
                        void* workspace, size_t workspace_bytes, void* stream);
+int jtmoe_moe_backward_sf(const void* x, const void* dy, const float* d_scores,
+                          const void* w_router, const void* gate, const void* up, const void* down,
+                          const void* shared_gate, const void* shared_up, const void* shared_down,
+                          const float* scores, const int32_t* expert_ids, const void* weights,
+                          const int32_t* source_order, const int32_t* inverse,
+                          const int32_t* group_sizes, const int32_t* offsets,
+                          const void* gate_pre, const void* up_pre,
+                          const void* shared_gate_pre, const void* shared_up_pre,
+                          double route_scale, int score_func,
+                          int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype,
+                          void* dx, void* d_w_router, void* d_gate, void* d_up, void* d_down,
+                          void* d_shared_gate, void* d_shared_up, void* d_shared_down,
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

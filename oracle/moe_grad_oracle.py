@@ -118,22 +118,35 @@ class RouterGrad:
     d_logits: np.ndarray  # [T,E]
 
 
-def router_backward(x, w_router, expert_ids, d_weights, d_scores, route_scale, scores=None) -> RouterGrad:
-    """Gradient of weights = scale * p / (sum p + 1e-20), p = sigmoid(x W)[ids], plus a cotangent on the scores.
+def _softmax(z):
+    e = np.exp(z - z.max(-1, keepdims=True))
+    return e / e.sum(-1, keepdims=True)
 
-    ``scores`` overrides sigmoid(x W) (pass the forward's own scores to follow its rounding).
+
+def router_backward(x, w_router, expert_ids, d_weights, d_scores, route_scale, scores=None,
+                    score_func="sigmoid") -> RouterGrad:
+    """Gradient of weights = scale * p / (sum p + 1e-20), p = score(x W)[ids], plus a cotangent on the scores.
+    score = sigmoid (the reference's router) or softmax over the experts (the attribute this build adds).
+
+    ``scores`` overrides score(x W) (pass the forward's own scores to follow its rounding).
     """
     x, w_router, d_weights = _f64(x), _f64(w_router), _f64(d_weights)
     ids = np.asarray(expert_ids)
     T = x.shape[0]
-    sc = _sigmoid(x @ w_router) if scores is None else _f64(scores)
+    if scores is not None:
+        sc = _f64(scores)
+    else:
+        sc = _sigmoid(x @ w_router) if score_func == "sigmoid" else _softmax(x @ w_router)
     rows = np.arange(T)[:, None]
     p = sc[rows, ids]
     S = p.sum(-1, keepdims=True) + 1e-20
     dp = route_scale * (d_weights / S - np.sum(d_weights * p, axis=-1, keepdims=True) / S**2)
     d_sc = np.zeros_like(sc) if d_scores is None else _f64(d_scores).copy()
     np.add.at(d_sc, (np.broadcast_to(rows, ids.shape), ids), dp)
-    d_logits = d_sc * sc * (1.0 - sc)
+    if score_func == "sigmoid":
+        d_logits = d_sc * sc * (1.0 - sc)
+    else:  # softmax Jacobian: d z_e = s_e (g_e - sum_j g_j s_j)
+        d_logits = sc * (d_sc - np.sum(d_sc * sc, axis=-1, keepdims=True))
     return RouterGrad(d_logits @ w_router.T, x.T @ d_logits, d_logits)
 
 
@@ -149,13 +162,13 @@ class LayerGrad:
 
 
 def moe_backward(x, w_router, gate, up, down, shared, expert_ids, weights, dy, d_scores, route_scale,
-                 scores=None) -> LayerGrad:
+                 scores=None, score_func="sigmoid") -> LayerGrad:
     """Gradient of the layer y = routed(x) + shared(x) for the cotangents dy and d_scores.
 
     ``weights`` are the route weights the forward used; ``expert_ids`` its selection.
     """
     eg = experts_backward(x, expert_ids, weights, gate, up, down, dy)
-    rg = router_backward(x, w_router, expert_ids, eg.d_weights, d_scores, route_scale, scores)
+    rg = router_backward(x, w_router, expert_ids, eg.d_weights, d_scores, route_scale, scores, score_func)
     dx = eg.dx + rg.dx
     d_shared = None
     if shared is not None:

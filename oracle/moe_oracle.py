@@ -41,6 +41,8 @@ Parity status of each function (what pins it is exercised in
   top-k with deliberately tied scores.
 * top-k behaviour on NaN / Inf scores: PARITY UNPINNED (nothing in the
   reference's tests reaches it; inputs of every configuration are finite).
+* the softmax score function (``softmax_f32``, ``score_func="softmax"``): PARITY UNPINNED
+  against the reference, which has no such router; pinned by float64 closed forms only.
 * dispatch: pinned by ``np.bincount`` / ``np.cumsum`` / stable ``np.argsort``, a
   closed-form rank, permutation invariants and the reference's edge patterns
   (test_model.py:580-587).
@@ -158,6 +160,34 @@ def sigmoid_f32(z: np.ndarray) -> np.ndarray:
     return (F32(1.0) / (F32(1.0) + e)).astype(np.float32)
 
 
+def softmax_f32(logits: np.ndarray) -> np.ndarray:
+    """softmax over the last axis in float32 by a fixed sequence of operations.
+
+    The reference has no softmax router (moe.py:133 is a sigmoid); the benchmark's second
+    configuration names one, so it is offered as a score function of the same router and restated
+    here only from its definition: m = max_e z_e;  p_e = exp(max(z_e - m, -86));  the p_e are added
+    in four runs of ceil(E/4) consecutive experts, each run in index order, the four run sums as
+    (s0 + s1) + (s2 + s3);  score_e = p_e / sum.  PARITY UNPINNED against any reference
+    implementation; pinned here by float64 closed forms (tests/test_oracle_router.py).
+    """
+    z = np.asarray(logits, dtype=np.float32)
+    num_experts = z.shape[-1]
+    m = np.max(z, axis=-1, keepdims=True)
+    p = exp_f32(np.maximum(z - m, -_EXP_CLAMP))
+    run = (num_experts + 3) // 4
+    sums = []
+    for q in range(4):
+        acc = np.zeros(z.shape[:-1], dtype=np.float32)
+        for e in range(q * run, min(num_experts, (q + 1) * run)):
+            acc = acc + p[..., e]
+        sums.append(acc)
+    total = (sums[0] + sums[1]) + (sums[2] + sums[3])
+    return (p / total[..., None]).astype(np.float32)
+
+
+SCORE_FUNCS = ("sigmoid", "softmax")
+
+
 def silu_f32(z: np.ndarray) -> np.ndarray:
     """z * sigmoid(z) in float32 (plain libm exp; outputs are tolerance-checked)."""
     z = np.asarray(z, dtype=np.float32)
@@ -195,15 +225,19 @@ def router_from_logits(
     top_k: int,
     route_scale: float,
     dtype: str,
+    score_func: str = "sigmoid",
 ) -> RouterResult:
-    """Everything after the projection (moe.py:133-147)."""
+    """Everything after the projection (moe.py:133-147).  score_func "softmax" replaces the sigmoid of
+    moe.py:133 by softmax_f32 and leaves the rest as it is (not a reference path)."""
     logits = np.asarray(logits, dtype=np.float32)
     num_experts = logits.shape[-1]
     if top_k <= 0 or top_k > num_experts:
         raise ValueError("router top_k must be positive and <= num_experts")
     if route_scale <= 0.0:
         raise ValueError("router route_scale must be positive")
-    scores = sigmoid_f32(logits)
+    if score_func not in SCORE_FUNCS:
+        raise ValueError(f"router score_func must be one of {SCORE_FUNCS}")
+    scores = sigmoid_f32(logits) if score_func == "sigmoid" else softmax_f32(logits)
     if expert_bias is None:
         expert_bias = np.zeros((num_experts,), dtype=np.float32)
     expert_bias = np.asarray(expert_bias, dtype=np.float32)
@@ -231,9 +265,10 @@ def router(
     top_k: int,
     route_scale: float = 1.0,
     dtype: str = "f32",
+    score_func: str = "sigmoid",
 ) -> RouterResult:
     """x [T,H], w_router [H,E] -> ids, weights, scores."""
-    return router_from_logits(router_logits(x, w_router, dtype), expert_bias, top_k, route_scale, dtype)
+    return router_from_logits(router_logits(x, w_router, dtype), expert_bias, top_k, route_scale, dtype, score_func)
 
 
 # --------------------------------------------------------------------------
@@ -528,12 +563,13 @@ def moe_forward(
     dtype: str = "f32",
     shared: tuple[np.ndarray, np.ndarray, np.ndarray] | None = None,
     with_aux_loss: bool = False,
+    score_func: str = "sigmoid",
 ) -> MoeResult:
     """Expert-major formulation of the whole layer; x [B,S,H]."""
     batch, seq_len, hidden = x.shape
     num_experts = gate.shape[0]
     x2 = np.asarray(x, dtype=np.float32).reshape(batch * seq_len, hidden)
-    route = router(x2, w_router, expert_bias, top_k, route_scale, dtype)
+    route = router(x2, w_router, expert_bias, top_k, route_scale, dtype, score_func)
     disp = dispatch(route.expert_ids, num_experts, cast_compute(x2, dtype))
     packed_y = grouped_swiglu(disp.packed_x, gate, up, down, disp.group_sizes, dtype)
     shared_y = None

@@ -32,9 +32,19 @@ PROTOTYPES: dict[str, tuple] = {
         [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_dbl, c_int,
          c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr],
     ),
+    "jtmoe_router_sf": (
+        c_int,
+        [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_dbl, c_int, c_int,
+         c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr],
+    ),
     "jtmoe_router_from_logits": (
         c_int,
         [c_ptr, c_ptr, c_i64, c_i64, c_i64, c_dbl, c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr],
+    ),
+    "jtmoe_router_from_logits_sf": (
+        c_int,
+        [c_ptr, c_ptr, c_i64, c_i64, c_i64, c_dbl, c_int, c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_size,
+         c_ptr],
     ),
     "jtmoe_dispatch_workspace_bytes": (c_size, [c_i64, c_i64]),
     "jtmoe_dispatch": (
@@ -66,6 +76,10 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_ptr] * 9 + [c_i64] * 6 + [c_dbl, c_int] + [c_ptr] * 10 + [c_ptr, c_size, c_ptr],
     ),
+    "jtmoe_moe_forward_sf": (
+        c_int,
+        [c_ptr] * 9 + [c_i64] * 6 + [c_dbl, c_int, c_int] + [c_ptr] * 10 + [c_ptr, c_size, c_ptr],
+    ),
     "jtmoe_rmsnorm": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_dbl, c_int, c_ptr, c_ptr]),
     "jtmoe_combine_norm_residual": (
         c_int,
@@ -93,14 +107,26 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_ptr] * 6 + [c_dbl] + [c_i64] * 4 + [c_int] + [c_ptr] * 2 + [c_ptr, c_size, c_ptr],
     ),
+    "jtmoe_router_backward_sf": (
+        c_int,
+        [c_ptr] * 6 + [c_dbl, c_int] + [c_i64] * 4 + [c_int] + [c_ptr] * 2 + [c_ptr, c_size, c_ptr],
+    ),
     "jtmoe_moe_forward_train": (
         c_int,
         [c_ptr] * 9 + [c_i64] * 6 + [c_dbl, c_int] + [c_ptr] * 14 + [c_ptr, c_size, c_ptr],
+    ),
+    "jtmoe_moe_forward_train_sf": (
+        c_int,
+        [c_ptr] * 9 + [c_i64] * 6 + [c_dbl, c_int, c_int] + [c_ptr] * 14 + [c_ptr, c_size, c_ptr],
     ),
     "jtmoe_moe_backward_workspace_bytes": (c_size, [c_i64] * 6 + [c_int]),
     "jtmoe_moe_backward": (
         c_int,
         [c_ptr] * 21 + [c_dbl] + [c_i64] * 6 + [c_int] + [c_ptr] * 8 + [c_ptr, c_size, c_ptr],
+    ),
+    "jtmoe_moe_backward_sf": (
+        c_int,
+        [c_ptr] * 21 + [c_dbl, c_int] + [c_i64] * 6 + [c_int] + [c_ptr] * 8 + [c_ptr, c_size, c_ptr],
     ),
     "jtmoe_moe_forward_timed": (
         c_int,

@@ -20,11 +20,12 @@ class MoeLayerFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w_router, gate, up, down, shared_gate, shared_up, shared_down, expert_bias, top_k,
-                route_scale):
+                route_scale, score_func="sigmoid"):
         shared = None if shared_gate is None else (shared_gate, shared_up, shared_down)
         result, residuals = grad.moe_forward_train(x, w_router, expert_bias, gate, up, down, top_k, route_scale,
-                                                   shared=shared)
+                                                   shared=shared, score_func=score_func)
         ctx.route_scale = route_scale
+        ctx.score_func = score_func
         ctx.has_shared = shared is not None
         # Everything the backward pass reads goes through save_for_backward (which knows how to hold an
         # output such as the scores without a reference cycle); y itself is not needed again.
@@ -51,15 +52,16 @@ class MoeLayerFunction(torch.autograd.Function):
         if dy is None:
             dy = torch.zeros_like(x)
         g = grad.moe_backward(x, dy.contiguous(), None if d_scores is None else d_scores.contiguous(), w_router, gate,
-                              up, down, shared, result, residuals, ctx.route_scale)
+                              up, down, shared, result, residuals, ctx.route_scale, score_func=ctx.score_func)
         ds = g.d_shared if g.d_shared is not None else (None, None, None)
-        return g.dx, g.d_w_router, g.d_gate, g.d_up, g.d_down, ds[0], ds[1], ds[2], None, None, None
+        return g.dx, g.d_w_router, g.d_gate, g.d_up, g.d_down, ds[0], ds[1], ds[2], None, None, None, None
 
 
-def moe_layer(x, w_router, expert_bias, gate, up, down, top_k, route_scale=1.0, shared=None):
+def moe_layer(x, w_router, expert_bias, gate, up, down, top_k, route_scale=1.0, shared=None, score_func="sigmoid"):
     """Differentiable layer on x [T,H]: returns (y [T,H], scores [T,E] float32, expert_ids [T,K] int32)."""
     sg, su, sd = shared if shared is not None else (None, None, None)
-    return MoeLayerFunction.apply(x, w_router, gate, up, down, sg, su, sd, expert_bias, top_k, float(route_scale))
+    return MoeLayerFunction.apply(x, w_router, gate, up, down, sg, su, sd, expert_bias, top_k, float(route_scale),
+                                  score_func)
 
 
 class SequenceBalanceLossFunction(torch.autograd.Function):

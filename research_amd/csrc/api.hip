@@ -437,7 +437,8 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
                             int32_t* offsets, int32_t* source_order, int32_t* inverse, void* workspace,
                             size_t workspace_bytes, void* stream, void* gate_pre, void* up_pre,
                             void* shared_gate_pre, void* shared_up_pre, const void* residual = nullptr,
-                            const float* post_scale = nullptr, double eps = 0.0) {
+                            const float* post_scale = nullptr, double eps = 0.0,
+                            int score_func = JTMOE_SCORE_SIGMOID) {
   clear_error();
   const bool train = gate_pre != nullptr;
   JT_REQUIRE(dtype_ok(dtype), "moe_forward: unknown dtype %d", dtype);
@@ -456,7 +457,7 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
   bool stats_done = false, plan_done = false;
   int rc = router_for_layer(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
                             expert_counts, importance, group_sizes, offsets, source_order, inverse, w.router,
-                            w.router_bytes, &stats_done, &plan_done, as_stream(stream));
+                            w.router_bytes, score_func, &stats_done, &plan_done, as_stream(stream));
   if (rc) return rc;
   stage_mark(kStageRouter, as_stream(stream));
   // where the GEMM can apply the permutation while it fetches its A tiles, the permuted copy of
@@ -509,6 +510,19 @@ extern "C" int jtmoe_moe_forward(const void* x, const void* w_router, const floa
                           nullptr, nullptr, nullptr);
 }
 
+extern "C" int jtmoe_moe_forward_sf(const void* x, const void* w_router, const float* expert_bias, const void* gate,
+                                    const void* up, const void* down, const void* shared_gate, const void* shared_up,
+                                    const void* shared_down, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I,
+                                    int64_t Is, double route_scale, int score_func, int dtype, void* y,
+                                    int32_t* expert_ids, void* weights, float* scores, float* expert_counts,
+                                    float* importance, int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
+                                    int32_t* inverse, void* workspace, size_t workspace_bytes, void* stream) {
+  return moe_forward_impl(x, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H, E, K, I,
+                          Is, route_scale, dtype, y, expert_ids, weights, scores, expert_counts, importance,
+                          group_sizes, offsets, source_order, inverse, workspace, workspace_bytes, stream, nullptr,
+                          nullptr, nullptr, nullptr, nullptr, nullptr, 0.0, score_func);
+}
+
 extern "C" int jtmoe_moe_forward_train(const void* x, const void* w_router, const float* expert_bias,
                                        const void* gate, const void* up, const void* down, const void* shared_gate,
                                        const void* shared_up, const void* shared_down, int64_t T, int64_t H,
@@ -518,6 +532,21 @@ extern "C" int jtmoe_moe_forward_train(const void* x, const void* w_router, cons
                                        int32_t* offsets, int32_t* source_order, int32_t* inverse, void* gate_pre,
                                        void* up_pre, void* shared_gate_pre, void* shared_up_pre, void* workspace,
                                        size_t workspace_bytes, void* stream) {
+  return jtmoe_moe_forward_train_sf(x, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H,
+                                    E, K, I, Is, route_scale, JTMOE_SCORE_SIGMOID, dtype, y, expert_ids, weights, scores,
+                                    expert_counts, importance, group_sizes, offsets, source_order, inverse, gate_pre,
+                                    up_pre, shared_gate_pre, shared_up_pre, workspace, workspace_bytes, stream);
+}
+
+extern "C" int jtmoe_moe_forward_train_sf(const void* x, const void* w_router, const float* expert_bias,
+                                          const void* gate, const void* up, const void* down,
+                                          const void* shared_gate, const void* shared_up, const void* shared_down,
+                                          int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
+                                          double route_scale, int score_func, int dtype, void* y, int32_t* expert_ids,
+                                          void* weights, float* scores, float* expert_counts, float* importance,
+                                          int32_t* group_sizes, int32_t* offsets, int32_t* source_order,
+                                          int32_t* inverse, void* gate_pre, void* up_pre, void* shared_gate_pre,
+                                          void* shared_up_pre, void* workspace, size_t workspace_bytes, void* stream) {
   if (T > 0 && (gate_pre == nullptr || up_pre == nullptr || (Is > 0 && (!shared_gate_pre || !shared_up_pre)))) {
     clear_error();
     return fail(JTMOE_EINVAL, "moe_forward_train: null residual buffer");
@@ -526,7 +555,7 @@ extern "C" int jtmoe_moe_forward_train(const void* x, const void* w_router, cons
   return moe_forward_impl(x, w_router, expert_bias, gate, up, down, shared_gate, shared_up, shared_down, T, H, E, K, I,
                           Is, route_scale, dtype, y, expert_ids, weights, scores, expert_counts, importance,
                           group_sizes, offsets, source_order, inverse, workspace, workspace_bytes, stream,
-                          gate_pre, up_pre, shared_gate_pre, shared_up_pre);
+                          gate_pre, up_pre, shared_gate_pre, shared_up_pre, nullptr, nullptr, 0.0, score_func);
 }
 
 extern "C" size_t jtmoe_ffn_block_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,

@@ -156,7 +156,8 @@ __global__ __launch_bounds__(256) void router_backward_kernel(const float* __res
                                                               const int32_t* __restrict__ ids,
                                                               const T* __restrict__ d_weights,
                                                               const float* __restrict__ d_scores, float route_scale,
-                                                              int tokens, int E, int K, T* __restrict__ d_logits) {
+                                                              int tokens, int E, int K, T* __restrict__ d_logits,
+                                                              int score_func) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= tokens) return;
   const int lane = threadIdx.x & 63;
@@ -171,10 +172,24 @@ __global__ __launch_bounds__(256) void router_backward_kernel(const float* __res
   }
   S += 1e-20f;
   const float c = dot / (S * S);
-  for (int e = lane; e < E; e += 64) {
+  // gradient with respect to the score of expert e (lane e, e + 64, ...)
+  auto score_grad = [&](int e) {
     float ds = d_scores ? d_scores[(size_t)t * E + e] : 0.0f;
     for (int s = 0; s < K; ++s)
       if (ids[(size_t)t * K + s] == e) ds += route_scale * (Elem<T>::load(d_weights + (size_t)t * K + s) / S - c);
+    return ds;
+  };
+  if (score_func == JTMOE_SCORE_SOFTMAX) {
+    // softmax over the experts: d z_e = p_e (g_e - sum_j g_j p_j); the sum by lane, then across the wave
+    float inner = 0.0f;
+    for (int e = lane; e < E; e += 64) inner += score_grad(e) * sc[e];
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) inner += __shfl_xor(inner, d);
+    for (int e = lane; e < E; e += 64) Elem<T>::store(d_logits + (size_t)t * E + e, sc[e] * (score_grad(e) - inner));
+    return;
+  }
+  for (int e = lane; e < E; e += 64) {
+    const float ds = score_grad(e);
     const float p = sc[e];
     Elem<T>::store(d_logits + (size_t)t * E + e, ds * p * (1.0f - p));
   }
@@ -335,7 +350,7 @@ int shared_backward_impl(const void* x, const void* dy, const void* gate, const 
 int router_backward_impl(const void* x, const void* router_weight, const float* scores, const int32_t* ids,
                          const void* d_weights, const float* d_scores, double route_scale, int64_t T, int64_t H,
                          int64_t E, int64_t K, int dtype, void* dx, void* d_router_weight, const RouterBwdWs& ws,
-                         hipStream_t s) {
+                         hipStream_t s, int score_func = JTMOE_SCORE_SIGMOID) {
   void* const d_logits = ws.d_logits;
   const unsigned grid = (unsigned)((T + 3) / 4);
   if (T == 0) {
@@ -343,11 +358,11 @@ int router_backward_impl(const void* x, const void* router_weight, const float* 
   } else if (dtype == JTMOE_BF16)
     router_backward_kernel<bf16_raw><<<grid, 256, 0, s>>>(scores, ids, static_cast<const bf16_raw*>(d_weights),
                                                           d_scores, (float)route_scale, (int)T, (int)E, (int)K,
-                                                          static_cast<bf16_raw*>(d_logits));
+                                                          static_cast<bf16_raw*>(d_logits), score_func);
   else
     router_backward_kernel<float><<<grid, 256, 0, s>>>(scores, ids, static_cast<const float*>(d_weights), d_scores,
                                                        (float)route_scale, (int)T, (int)E, (int)K,
-                                                       static_cast<float*>(d_logits));
+                                                       static_cast<float*>(d_logits), score_func);
   int rc = check_launch("router backward");
   if (rc) return rc;
   // dW_r [H, E] = x^T @ dlogits;  dx [T, H] = dlogits @ W_r^T  (W_r is [H, E]: N = H rows of length K = E)
@@ -468,9 +483,20 @@ extern "C" int jtmoe_router_backward(const void* x, const void* router_weight, c
                                      double route_scale, int64_t T, int64_t H, int64_t E, int64_t K, int dtype,
                                      void* dx, void* d_router_weight, void* workspace, size_t workspace_bytes,
                                      void* stream) {
+  return jtmoe_router_backward_sf(x, router_weight, scores, expert_ids, d_weights, d_scores, route_scale,
+                                  JTMOE_SCORE_SIGMOID, T, H, E, K, dtype, dx, d_router_weight, workspace,
+                                  workspace_bytes, stream);
+}
+
+extern "C" int jtmoe_router_backward_sf(const void* x, const void* router_weight, const float* scores,
+                                        const int32_t* expert_ids, const void* d_weights, const float* d_scores,
+                                        double route_scale, int score_func, int64_t T, int64_t H, int64_t E,
+                                        int64_t K, int dtype, void* dx, void* d_router_weight, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
   clear_error();
   int rc = validate_shape("router_backward", T, K, H, 1, E, dtype);
   if (rc) return rc;
+  JT_REQUIRE(score_func_ok(score_func), "router_backward: unknown score function %d", score_func);
   JT_REQUIRE(router_weight && d_router_weight, "router_backward: null weight pointer");
   if (T > 0) JT_REQUIRE(x && scores && expert_ids && d_weights && dx, "router_backward: null pointer argument");
   const RouterBwdWs ws = carve_router(workspace, T, H, E, dtype);
@@ -478,7 +504,7 @@ extern "C" int jtmoe_router_backward(const void* x, const void* router_weight, c
     return fail(JTMOE_EWORKSPACE, "router_backward: workspace of %zu bytes given, %zu needed", workspace_bytes,
                 ws.total);
   return router_backward_impl(x, router_weight, scores, expert_ids, d_weights, d_scores, route_scale, T, H, E, K,
-                              dtype, dx, d_router_weight, ws, as_stream(stream));
+                              dtype, dx, d_router_weight, ws, as_stream(stream), score_func);
 }
 
 extern "C" size_t jtmoe_moe_backward_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
@@ -502,9 +528,28 @@ extern "C" int jtmoe_moe_backward(const void* x, const void* dy, const float* d_
                                   int64_t K, int64_t I, int64_t Is, int dtype, void* dx, void* d_router_weight,
                                   void* d_gate, void* d_up, void* d_down, void* d_shared_gate, void* d_shared_up,
                                   void* d_shared_down, void* workspace, size_t workspace_bytes, void* stream) {
+  return jtmoe_moe_backward_sf(x, dy, d_scores, router_weight, gate, up, down, shared_gate, shared_up, shared_down,
+                               scores, expert_ids, weights, source_order, inverse, group_sizes, offsets, gate_pre,
+                               up_pre, shared_gate_pre, shared_up_pre, route_scale, JTMOE_SCORE_SIGMOID, T, H, E, K, I,
+                               Is, dtype, dx, d_router_weight, d_gate, d_up, d_down, d_shared_gate, d_shared_up,
+                               d_shared_down, workspace, workspace_bytes, stream);
+}
+
+extern "C" int jtmoe_moe_backward_sf(const void* x, const void* dy, const float* d_scores, const void* router_weight,
+                                     const void* gate, const void* up, const void* down, const void* shared_gate,
+                                     const void* shared_up, const void* shared_down, const float* scores,
+                                     const int32_t* expert_ids, const void* weights, const int32_t* source_order,
+                                     const int32_t* inverse, const int32_t* group_sizes, const int32_t* offsets,
+                                     const void* gate_pre, const void* up_pre, const void* shared_gate_pre,
+                                     const void* shared_up_pre, double route_scale, int score_func, int64_t T,
+                                     int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype, void* dx,
+                                     void* d_router_weight, void* d_gate, void* d_up, void* d_down,
+                                     void* d_shared_gate, void* d_shared_up, void* d_shared_down, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
   clear_error();
   int rc = validate_shape("moe_backward", T, K, H, I, E, dtype);
   if (rc) return rc;
+  JT_REQUIRE(score_func_ok(score_func), "moe_backward: unknown score function %d", score_func);
   JT_REQUIRE(Is >= 0, "moe_backward: Is=%lld out of range", (long long)Is);
   JT_REQUIRE(router_weight && gate && up && down && d_router_weight && d_gate && d_up && d_down,
              "moe_backward: null weight pointer");
@@ -541,7 +586,7 @@ extern "C" int jtmoe_moe_backward(const void* x, const void* dy, const float* d_
     if (rc) return rc;
   }
   rc = router_backward_impl(x, router_weight, scores, expert_ids, d_weights, d_scores, route_scale, T, H, E, K, dtype,
-                            dx_router, d_router_weight, rws, s);
+                            dx_router, d_router_weight, rws, s, score_func);
   if (rc) return rc;
   if (T == 0) return JTMOE_OK;
   const void* extra = dx_router;

@@ -19,6 +19,7 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline size_t dtype_bytes(int dtype) { return dtype == JTMOE_F32 ? 4 : 2; }
 inline bool dtype_ok(int dtype) { return dtype == JTMOE_BF16 || dtype == JTMOE_F32; }
+inline bool score_func_ok(int f) { return f == JTMOE_SCORE_SIGMOID || f == JTMOE_SCORE_SOFTMAX; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- optional per-stage timing (only jtmoe_moe_forward_timed installs a timer) ----
@@ -132,6 +133,6 @@ int router_for_layer(const void* x, const void* w_router, const float* expert_bi
                      int64_t K, double route_scale, int dtype, int32_t* expert_ids, void* weights, float* scores,
                      float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
                      int32_t* source_order, int32_t* inverse, void* workspace, size_t workspace_bytes,
-                     bool* stats_done, bool* plan_done, hipStream_t stream);
+                     int score_func, bool* stats_done, bool* plan_done, hipStream_t stream);
 
 }  // namespace jtmoe

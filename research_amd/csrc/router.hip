@@ -231,25 +231,62 @@ template <typename T, int kRouterTokens, int kRouterThreads>
 __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ bias_g, int t0, int tokens,
                                 int E, int K, float route_scale, int32_t* __restrict__ ids_out,
                                 T* __restrict__ weights_out, float* __restrict__ scores_out,
-                                float* __restrict__ logits_out, RouterScratch g,
+                                float* __restrict__ logits_out, RouterScratch g, int score_func,
                                 float* __restrict__ counts_final = nullptr,
                                 float* __restrict__ importance_final = nullptr) {
 #pragma clang fp contract(off)
   const int tid = threadIdx.x;
   const int stride = E + 1;
   const int nrows = min(kRouterTokens, tokens - t0);
+  const bool softmax = score_func == JTMOE_SCORE_SOFTMAX;
 
   for (int e = tid; e < E; e += kRouterThreads) {
     sm.bias[e] = bias_g ? bias_g[e] : 0.0f;
     sm.cnt[e] = 0;
     sm.imp[e] = 0ull;
   }
+  if (softmax) {
+    // Softmax over the experts of every token, in place, by the token's four lanes (lane q owns the
+    // run of ceil(E/4) consecutive experts that it owns in the selection below):
+    // m = max z;  p_e = exp(max(z_e - m, -86));  the four run sums, each added in index order, are
+    // combined as (s0 + s1) + (s2 + s3);  score_e = p_e / sum.  A fixed sequence of fp32 operations.
+    if (logits_out)
+      for (int idx = tid; idx < nrows * E; idx += kRouterThreads) {
+        const int t = idx / E, e = idx - t * E;
+        logits_out[(size_t)(t0 + t) * E + e] = sm.tile[t * stride + e];
+      }
+    __syncthreads();
+    const int t = tid >> 2, q = tid & 3;
+    const int eq = (E + 3) >> 2;
+    const int e_lo = q * eq, e_hi = min(E, e_lo + eq);
+    const bool row_ok = t < nrows;
+    float* const row = sm.tile + t * stride;
+    float m = -INFINITY;
+    if (row_ok)
+      for (int e = e_lo; e < e_hi; ++e) m = fmaxf(m, row[e]);
+    m = fmaxf(m, quad_xor_f32<1>(m));
+    m = fmaxf(m, quad_xor_f32<2>(m));
+    float part = 0.0f;
+    if (row_ok)
+      for (int e = e_lo; e < e_hi; ++e) {
+        float d = row[e] - m;
+        d = fmaxf(d, -86.0f);
+        const float p = exp_fixed(d);
+        row[e] = p;
+        part = part + p;
+      }
+    const float pair = part + quad_xor_f32<1>(part);
+    const float total = pair + quad_xor_f32<2>(pair);
+    if (row_ok)
+      for (int e = e_lo; e < e_hi; ++e) row[e] = row[e] / total;
+    __syncthreads();
+  }
   // logits -> scores (in place), both written out row-major
   for (int idx = tid; idx < nrows * E; idx += kRouterThreads) {
     const int t = idx / E, e = idx - t * E;
     const float z = sm.tile[t * stride + e];
-    if (logits_out) logits_out[(size_t)(t0 + t) * E + e] = z;
-    const float s = sigmoid_fixed(z);
+    if (logits_out && !softmax) logits_out[(size_t)(t0 + t) * E + e] = z;
+    const float s = softmax ? z : sigmoid_fixed(z);
     sm.tile[t * stride + e] = s;
     scores_out[(size_t)(t0 + t) * E + e] = s;
   }
@@ -316,7 +353,7 @@ __global__ __launch_bounds__(256) void router_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ logits_in,
     const float* __restrict__ bias, int tokens, int H, int E, int K, float route_scale,
     int32_t* __restrict__ ids, T* __restrict__ weights, float* __restrict__ scores,
-    float* __restrict__ logits_out, void* ws) {
+    float* __restrict__ logits_out, void* ws, int score_func) {
   constexpr int kRouterTokens = 64, kRouterThreads = 256;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   RouterSmem sm = router_smem(smem_raw, E, K, kRouterTokens);
@@ -338,7 +375,7 @@ __global__ __launch_bounds__(256) void router_kernel(
   }
   __syncthreads();
   router_epilogue<T, 64, 256>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
-                              router_scratch(ws, E));
+                              router_scratch(ws, E), score_func);
 }
 
 // ---------------------------------------------------------------------------
@@ -369,7 +406,7 @@ template <int NB, int NW>
 __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
     int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
-    float* __restrict__ scores, float* __restrict__ logits_out, void* ws) {
+    float* __restrict__ scores, float* __restrict__ logits_out, void* ws, int score_func) {
   constexpr int kRouterTokens = 16 * NW, kRouterThreads = 64 * NW;
   constexpr int E = NB * 16;
   constexpr int WS = E + 32;                      // LDS row stride of the staged matrix (elements)
@@ -512,7 +549,7 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
       sm.tile[(wave * 16 + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = round_to_bf16(acc[nb][i]);
   __syncthreads();
   router_epilogue<bf16_raw, 16 * NW, 64 * NW>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores,
-                                              logits_out, router_scratch(ws, E));
+                                              logits_out, router_scratch(ws, E), score_func);
 }
 
 // ---------------------------------------------------------------------------
@@ -542,7 +579,7 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
     int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
     float* __restrict__ scores, float* __restrict__ logits_out, void* ws, float* __restrict__ partial_out,
-    int chunks_per_slice) {
+    int chunks_per_slice, int score_func) {
   constexpr int kThreads = 256, kTokens = 16;
   constexpr int E = NB * 16;
   constexpr int WS = E + 32;
@@ -651,7 +688,7 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
   if (kPartial) return;
   __syncthreads();
   router_epilogue<bf16_raw, kTokens, kThreads>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores,
-                                               logits_out, router_scratch(ws, E));
+                                               logits_out, router_scratch(ws, E), score_func);
 }
 
 // Second half of the small-batch router: one workgroup adds the slices of partial sums in slice
@@ -669,7 +706,7 @@ __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
     float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights, float* __restrict__ scores,
     float* __restrict__ logits_out, float* __restrict__ counts, float* __restrict__ importance,
     int32_t* __restrict__ group_sizes, int32_t* __restrict__ offsets, int32_t* __restrict__ source_order,
-    int32_t* __restrict__ inverse) {
+    int32_t* __restrict__ inverse, int score_func) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   RouterSmem sm = router_smem(smem_raw, E, K, kTok);
   const int stride = E + 1;
@@ -688,7 +725,7 @@ __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
   }
   __syncthreads();
   router_epilogue<bf16_raw, kTok, 4 * kTok>(sm, bias, 0, tokens, E, K, route_scale, ids, weights, scores, logits_out,
-                                            RouterScratch{}, counts, importance);
+                                            RouterScratch{}, score_func, counts, importance);
   if (kPlan) {
     static_assert(kTok >= 1 + 4 * kTok / kWave, "the plan's tables fit into the score tile");
     dispatch_small_body<4 * kTok, false, bf16_raw>(sm.top_id, nullptr, tokens * K, E, group_sizes, offsets,
@@ -721,7 +758,7 @@ template <typename T, bool kFromLogits>
 int launch_router(const void* x, const void* w, const float* logits_in, const float* bias, int64_t tokens,
                   int64_t H, int64_t E, int64_t K, double route_scale, int32_t* ids, void* weights,
                   float* scores, float* counts, float* importance, float* logits_out, void* ws,
-                  hipStream_t stream, LayerPlan* layer = nullptr) {
+                  hipStream_t stream, int score_func, LayerPlan* layer = nullptr) {
   // a stand-alone call always computes the statistics; a layer call only where they cost no launch
   const bool stats = layer == nullptr;
   void* const ws_stats = stats ? ws : nullptr;
@@ -753,7 +790,8 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (rc) return rc;                                                                                       \
     kernel<<<dim3(blocks, slices), 256, smem, stream>>>(                                                     \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws, partial, per_slice); \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws, partial, per_slice, \
+        score_func);                                                                                         \
   } break;
         switch ((int)E) {
           JT_PARTIAL_CASE(1)
@@ -774,7 +812,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
                                           ids, static_cast<bf16_raw*>(weights), scores, logits_out, counts,        \
                                           importance, PLAN ? layer->group_sizes : nullptr,                         \
                                           PLAN ? layer->offsets : nullptr, PLAN ? layer->source_order : nullptr,   \
-                                          PLAN ? layer->inverse : nullptr);                                        \
+                                          PLAN ? layer->inverse : nullptr, score_func);                            \
   }
         if (finish_tok == 256) {
           if (plan) JT_FINISH(256, true) else JT_FINISH(256, false)
@@ -797,7 +835,8 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (rc) return rc;                                                                                       \
     kernel<<<blocks, 256, smem, stream>>>(                                                                   \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats, nullptr, 0); \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats, nullptr, 0,  \
+        score_func);                                                                                         \
   } break;
         switch ((int)E) {
           JT_SPLIT_CASE(1)
@@ -827,7 +866,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (rc) return rc;                                                                                       \
     kernel<<<blocks, 64 * NW, smem, stream>>>(                                                               \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats);             \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats, score_func); \
   }
 #define JT_ROUTER_CASE(NB)    \
   case NB * 16:               \
@@ -854,7 +893,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (tokens > 0)
       kernel<<<blocks, 256, smem, stream>>>(
           static_cast<const T*>(x), static_cast<const T*>(w), logits_in, bias, (int)tokens, (int)H, (int)E, (int)K,
-          (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws_stats);
+          (float)route_scale, ids, static_cast<T*>(weights), scores, logits_out, ws_stats, score_func);
   }
   if (stats) router_finalize_kernel<<<1, 256, 0, stream>>>(ws, (int)E, counts, importance);
   return check_launch("router");
@@ -879,9 +918,10 @@ int router_for_layer(const void* x, const void* w_router, const float* expert_bi
                      int64_t K, double route_scale, int dtype, int32_t* expert_ids, void* weights, float* scores,
                      float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
                      int32_t* source_order, int32_t* inverse, void* workspace, size_t workspace_bytes,
-                     bool* stats_done, bool* plan_done, hipStream_t s) {
+                     int score_func, bool* stats_done, bool* plan_done, hipStream_t s) {
   int rc = validate_router(T, H, E, K, route_scale, dtype, true);
   if (rc) return rc;
+  JT_REQUIRE(score_func_ok(score_func), "router: unknown score function %d", score_func);
   JT_REQUIRE(w_router && expert_counts && importance && workspace, "router: null pointer argument");
   JT_REQUIRE(T == 0 || (x && expert_ids && weights && scores), "router: null pointer argument");
   JT_REQUIRE(group_sizes && offsets && (T == 0 || (source_order && inverse)), "router: null pointer argument");
@@ -890,10 +930,10 @@ int router_for_layer(const void* x, const void* w_router, const float* expert_bi
   LayerPlan layer{group_sizes, offsets, source_order, inverse, false, false};
   if (dtype == JTMOE_BF16)
     rc = launch_router<bf16_raw, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
-                                        scores, expert_counts, importance, nullptr, workspace, s, &layer);
+                                        scores, expert_counts, importance, nullptr, workspace, s, score_func, &layer);
   else
     rc = launch_router<float, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
-                                     scores, expert_counts, importance, nullptr, workspace, s, &layer);
+                                     scores, expert_counts, importance, nullptr, workspace, s, score_func, &layer);
   *stats_done = layer.stats_done;
   *plan_done = layer.plan_done;
   return rc;
@@ -913,9 +953,19 @@ extern "C" int jtmoe_router(const void* x, const void* w_router, const float* ex
                             int64_t E, int64_t K, double route_scale, int dtype, int32_t* expert_ids,
                             void* weights, float* scores, float* expert_counts, float* importance, float* logits,
                             void* workspace, size_t workspace_bytes, void* stream) {
+  return jtmoe_router_sf(x, w_router, expert_bias, T, H, E, K, route_scale, JTMOE_SCORE_SIGMOID, dtype, expert_ids,
+                         weights, scores, expert_counts, importance, logits, workspace, workspace_bytes, stream);
+}
+
+extern "C" int jtmoe_router_sf(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H,
+                               int64_t E, int64_t K, double route_scale, int score_func, int dtype,
+                               int32_t* expert_ids, void* weights, float* scores, float* expert_counts,
+                               float* importance, float* logits, void* workspace, size_t workspace_bytes,
+                               void* stream) {
   clear_error();
   int rc = validate_router(T, H, E, K, route_scale, dtype, true);
   if (rc) return rc;
+  JT_REQUIRE(score_func_ok(score_func), "router: unknown score function %d", score_func);
   JT_REQUIRE(w_router && expert_counts && importance && workspace, "router: null pointer argument");
   JT_REQUIRE(T == 0 || (x && expert_ids && weights && scores), "router: null pointer argument");
   if (workspace_bytes < jtmoe_router_workspace_bytes(E))
@@ -923,18 +973,28 @@ extern "C" int jtmoe_router(const void* x, const void* w_router, const float* ex
   hipStream_t s = as_stream(stream);
   if (dtype == JTMOE_BF16)
     return launch_router<bf16_raw, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids,
-                                          weights, scores, expert_counts, importance, logits, workspace, s);
+                                          weights, scores, expert_counts, importance, logits, workspace, s, score_func);
   return launch_router<float, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
-                                     scores, expert_counts, importance, logits, workspace, s);
+                                     scores, expert_counts, importance, logits, workspace, s, score_func);
 }
 
 extern "C" int jtmoe_router_from_logits(const float* logits, const float* expert_bias, int64_t T, int64_t E,
                                         int64_t K, double route_scale, int dtype, int32_t* expert_ids,
                                         void* weights, float* scores, float* expert_counts, float* importance,
                                         void* workspace, size_t workspace_bytes, void* stream) {
+  return jtmoe_router_from_logits_sf(logits, expert_bias, T, E, K, route_scale, JTMOE_SCORE_SIGMOID, dtype, expert_ids,
+                                     weights, scores, expert_counts, importance, workspace, workspace_bytes, stream);
+}
+
+extern "C" int jtmoe_router_from_logits_sf(const float* logits, const float* expert_bias, int64_t T, int64_t E,
+                                           int64_t K, double route_scale, int score_func, int dtype,
+                                           int32_t* expert_ids, void* weights, float* scores, float* expert_counts,
+                                           float* importance, void* workspace, size_t workspace_bytes,
+                                           void* stream) {
   clear_error();
   int rc = validate_router(T, 1, E, K, route_scale, dtype, false);
   if (rc) return rc;
+  JT_REQUIRE(score_func_ok(score_func), "router_from_logits: unknown score function %d", score_func);
   JT_REQUIRE(expert_counts && importance && workspace, "router_from_logits: null pointer argument");
   JT_REQUIRE(T == 0 || (logits && expert_ids && weights && scores), "router_from_logits: null pointer argument");
   if (workspace_bytes < jtmoe_router_workspace_bytes(E))
@@ -943,7 +1003,7 @@ extern "C" int jtmoe_router_from_logits(const float* logits, const float* expert
   hipStream_t s = as_stream(stream);
   if (dtype == JTMOE_BF16)
     return launch_router<bf16_raw, true>(nullptr, nullptr, logits, expert_bias, T, 0, E, K, route_scale, expert_ids,
-                                         weights, scores, expert_counts, importance, nullptr, workspace, s);
+                                         weights, scores, expert_counts, importance, nullptr, workspace, s, score_func);
   return launch_router<float, true>(nullptr, nullptr, logits, expert_bias, T, 0, E, K, route_scale, expert_ids, weights,
-                                    scores, expert_counts, importance, nullptr, workspace, s);
+                                    scores, expert_counts, importance, nullptr, workspace, s, score_func);
 }

@@ -154,7 +154,8 @@ def shared_backward(x, dy, gate, up, down, residuals: ExpertResiduals):
     return dx, d_gate, d_up, d_down
 
 
-def router_backward(x, w_router, scores, expert_ids, d_weights, d_scores=None, route_scale: float = 1.0):
+def router_backward(x, w_router, scores, expert_ids, d_weights, d_scores=None, route_scale: float = 1.0,
+                    score_func: str = "sigmoid"):
     """VJP of the router for the cotangents d_weights [T,K] and (optionally) d_scores [T,E]: (dx, d_w_router)."""
     _check(x, "x")
     if x.dim() != 2:
@@ -177,10 +178,12 @@ def router_backward(x, w_router, scores, expert_ids, d_weights, d_scores=None, r
     d_w = torch.empty_like(w_router)
     lib = _lib()
     ws = _workspace(lib.jtmoe_router_backward_workspace_bytes(tokens, hidden, experts, _code(x.dtype)), dev)
-    status = lib.jtmoe_router_backward(
-        _ptr(x), _ptr(w_router), _ptr(scores), _ptr(expert_ids), _ptr(d_weights), _ptr(d_scores), float(route_scale),
-        tokens, hidden, experts, top_k, _code(x.dtype), _ptr(dx), _ptr(d_w), ws.data_ptr(), ws.numel(), _stream(dev),
-    )
+    head = (_ptr(x), _ptr(w_router), _ptr(scores), _ptr(expert_ids), _ptr(d_weights), _ptr(d_scores),
+            float(route_scale))
+    tail = (tokens, hidden, experts, top_k, _code(x.dtype), _ptr(dx), _ptr(d_w), ws.data_ptr(), ws.numel(),
+            _stream(dev))
+    code = ops._score_code(score_func)
+    status = lib.jtmoe_router_backward(*head, *tail) if code == 0 else lib.jtmoe_router_backward_sf(*head, code, *tail)
     _raise(status, "jtmoe_router_backward")
     return dx, d_w
 
@@ -201,7 +204,8 @@ class LayerGrad:
     d_shared: tuple | None
 
 
-def moe_forward_train(x, w_router, expert_bias, gate, up, down, top_k, route_scale: float = 1.0, shared=None):
+def moe_forward_train(x, w_router, expert_bias, gate, up, down, top_k, route_scale: float = 1.0, shared=None,
+                      score_func: str = "sigmoid"):
     """The layer forward through jtmoe_moe_forward_train: (ops.LayerResult, LayerResiduals)."""
     tokens, hidden, experts, inter = _expert_shapes(x, gate, up, down)
     _check(w_router, "w_router", x.dtype, (hidden, experts))
@@ -235,15 +239,19 @@ def moe_forward_train(x, w_router, expert_bias, gate, up, down, top_k, route_sca
     lib = _lib()
     nbytes = lib.jtmoe_workspace_bytes(tokens, hidden, experts, top_k, inter, shared_inter, _code(x.dtype))
     ws = ops.layer_workspace(nbytes, dev)
-    status = lib.jtmoe_moe_forward_train(
-        _ptr(x), _ptr(w_router), _ptr(expert_bias), _ptr(gate), _ptr(up), _ptr(down), _ptr(sg), _ptr(su), _ptr(sd),
-        tokens, hidden, experts, top_k, inter, shared_inter, float(route_scale), _code(x.dtype),
+    head = (_ptr(x), _ptr(w_router), _ptr(expert_bias), _ptr(gate), _ptr(up), _ptr(down), _ptr(sg), _ptr(su), _ptr(sd),
+            tokens, hidden, experts, top_k, inter, shared_inter, float(route_scale))
+    tail = (
+        _code(x.dtype),
         _ptr(y), _ptr(expert_ids), _ptr(weights), _ptr(scores), _ptr(expert_counts), _ptr(importance),
         _ptr(group_sizes), _ptr(offsets), _ptr(source_order), _ptr(inverse),
         _ptr(routed.gate_pre), _ptr(routed.up_pre),
         _ptr(shared_res.gate_pre) if shared_res else None, _ptr(shared_res.up_pre) if shared_res else None,
         ws.data_ptr(), ws.numel(), _stream(dev),
     )
+    code = ops._score_code(score_func)
+    status = (lib.jtmoe_moe_forward_train(*head, *tail) if code == 0
+              else lib.jtmoe_moe_forward_train_sf(*head, code, *tail))
     _raise(status, "jtmoe_moe_forward_train")
     result = ops.LayerResult(y, expert_ids, weights, scores, expert_counts, importance, group_sizes, offsets,
                              source_order, inverse)
@@ -254,7 +262,7 @@ _BACKWARD_WORKSPACES: dict[tuple, torch.Tensor] = {}
 
 
 def moe_backward(x, dy, d_scores, w_router, gate, up, down, shared, result: ops.LayerResult,
-                 residuals: LayerResiduals, route_scale: float = 1.0) -> LayerGrad:
+                 residuals: LayerResiduals, route_scale: float = 1.0, score_func: str = "sigmoid") -> LayerGrad:
     """VJP of the layer for the cotangents dy [T,H] and d_scores [T,E] (or None)."""
     tokens, hidden, experts, inter = _expert_shapes(x, gate, up, down)
     _check(dy, "dy", x.dtype, (tokens, hidden))
@@ -283,17 +291,22 @@ def moe_backward(x, dy, d_scores, w_router, gate, up, down, shared, result: ops.
         ws = _workspace(nbytes, dev)
         _BACKWARD_WORKSPACES[key] = ws
     sres = residuals.shared
-    status = lib.jtmoe_moe_backward(
+    head = (
         _ptr(x), _ptr(dy), _ptr(d_scores), _ptr(w_router), _ptr(gate), _ptr(up), _ptr(down),
         _ptr(sg), _ptr(su), _ptr(sd), _ptr(result.scores), _ptr(result.expert_ids), _ptr(result.weights),
         _ptr(result.source_order), _ptr(result.inverse), _ptr(result.group_sizes), _ptr(result.offsets),
         _ptr(residuals.routed.gate_pre), _ptr(residuals.routed.up_pre),
         _ptr(sres.gate_pre) if sres else None, _ptr(sres.up_pre) if sres else None,
-        float(route_scale), tokens, hidden, experts, top_k, inter, shared_inter, _code(x.dtype),
+        float(route_scale),
+    )
+    tail = (
+        tokens, hidden, experts, top_k, inter, shared_inter, _code(x.dtype),
         _ptr(dx), _ptr(d_w), _ptr(d_gate), _ptr(d_up), _ptr(d_down),
         _ptr(d_shared[0]) if d_shared else None, _ptr(d_shared[1]) if d_shared else None,
         _ptr(d_shared[2]) if d_shared else None,
         ws.data_ptr(), ws.numel(), _stream(dev),
     )
+    code = ops._score_code(score_func)
+    status = lib.jtmoe_moe_backward(*head, *tail) if code == 0 else lib.jtmoe_moe_backward_sf(*head, code, *tail)
     _raise(status, "jtmoe_moe_backward")
     return LayerGrad(dx, d_w, d_gate, d_up, d_down, d_shared)

@@ -77,6 +77,16 @@ class RouterResult:
     logits: torch.Tensor | None  # [T,E] float32 when requested
 
 
+SCORE_FUNCS = {"sigmoid": 0, "softmax": 1}  # JTMOE_SCORE_SIGMOID / JTMOE_SCORE_SOFTMAX of include/jtmoe.h
+
+
+def _score_code(score_func: str) -> int:
+    """"sigmoid" is the reference's router (moe.py:133); "softmax" is the attribute this library adds."""
+    if score_func not in SCORE_FUNCS:
+        raise ContractError(f"router score_func must be one of {sorted(SCORE_FUNCS)}, got {score_func!r}")
+    return SCORE_FUNCS[score_func]
+
+
 def _validate_router_attrs(num_experts: int, top_k: int, route_scale: float) -> None:
     if top_k <= 0 or num_experts <= 0 or top_k > num_experts:
         raise ContractError("router top_k must be positive and <= num_experts")
@@ -92,6 +102,7 @@ def router(
     route_scale: float = 1.0,
     *,
     return_logits: bool = False,
+    score_func: str = "sigmoid",
 ) -> RouterResult:
     """x [T,H], w_router [H,E] -> ids, weights, scores, counts, importance."""
     _check(x, "x")
@@ -117,11 +128,13 @@ def router(
     lib = _lib()
     ws_bytes = lib.jtmoe_router_workspace_bytes(experts)
     ws = _workspace(ws_bytes, dev)
-    status = lib.jtmoe_router(
-        _ptr(x), _ptr(w_router), _ptr(expert_bias), tokens, hidden, experts, top_k, float(route_scale),
-        _code(x.dtype), _ptr(ids), _ptr(weights), _ptr(scores), _ptr(counts), _ptr(importance), _ptr(logits),
-        _ptr(ws), ws.numel(), _stream(dev),
-    )
+    head = (_ptr(x), _ptr(w_router), _ptr(expert_bias), tokens, hidden, experts, top_k, float(route_scale))
+    tail = (_code(x.dtype), _ptr(ids), _ptr(weights), _ptr(scores), _ptr(counts), _ptr(importance), _ptr(logits),
+            _ptr(ws), ws.numel(), _stream(dev))
+    if _score_code(score_func) == 0:  # the reference's router: the entry point that replaces it
+        status = lib.jtmoe_router(*head, *tail)
+    else:
+        status = lib.jtmoe_router_sf(*head, _score_code(score_func), *tail)
     _raise(status, "jtmoe_router")
     return RouterResult(ids, weights, scores, counts, importance, logits)
 
@@ -133,6 +146,7 @@ def router_from_logits(
     route_scale: float = 1.0,
     *,
     dtype: torch.dtype = torch.float32,
+    score_func: str = "sigmoid",
 ) -> RouterResult:
     """Routing decision from given fp32 logits [T,E]; weights are cast to ``dtype``."""
     _check(logits, "logits", torch.float32)
@@ -152,10 +166,13 @@ def router_from_logits(
     importance = torch.empty((experts,), dtype=torch.float32, device=dev)
     lib = _lib()
     ws = _workspace(lib.jtmoe_router_workspace_bytes(experts), dev)
-    status = lib.jtmoe_router_from_logits(
-        _ptr(logits), _ptr(expert_bias), tokens, experts, top_k, float(route_scale), _code(dtype),
-        _ptr(ids), _ptr(weights), _ptr(scores), _ptr(counts), _ptr(importance), _ptr(ws), ws.numel(), _stream(dev),
-    )
+    head = (_ptr(logits), _ptr(expert_bias), tokens, experts, top_k, float(route_scale))
+    tail = (_code(dtype), _ptr(ids), _ptr(weights), _ptr(scores), _ptr(counts), _ptr(importance), _ptr(ws), ws.numel(),
+            _stream(dev))
+    if _score_code(score_func) == 0:
+        status = lib.jtmoe_router_from_logits(*head, *tail)
+    else:
+        status = lib.jtmoe_router_from_logits_sf(*head, _score_code(score_func), *tail)
     _raise(status, "jtmoe_router_from_logits")
     return RouterResult(ids, weights, scores, counts, importance, None)
 
@@ -490,8 +507,10 @@ def moe_forward(
     workspace: torch.Tensor | None = None,
     stage_ms: list | None = None,
     expert_counts_out: torch.Tensor | None = None,
+    score_func: str = "sigmoid",
 ) -> LayerResult:
-    """The whole layer on x [T,H] through the single C entry point jtmoe_moe_forward.
+    """The whole layer on x [T,H] through the single C entry point jtmoe_moe_forward
+    (jtmoe_moe_forward_sf for a score function other than the reference's sigmoid).
 
     ``expert_counts_out`` ([experts] f32, contiguous — e.g. one row of the [layers, experts] buffer
     the balancing update reads) receives the expert counts instead of a fresh tensor.
@@ -561,7 +580,11 @@ def moe_forward(
         _ptr(group_sizes), _ptr(offsets), _ptr(source_order), _ptr(inverse),
         workspace.data_ptr(), workspace.numel(), _stream(dev),
     )
-    if stage_ms is None:
+    if _score_code(score_func) != 0:
+        if stage_ms is not None:
+            raise ContractError("the per-stage timing entry point runs the reference's sigmoid router only")
+        status = lib.jtmoe_moe_forward_sf(*args[:16], _score_code(score_func), *args[16:])
+    elif stage_ms is None:
         status = lib.jtmoe_moe_forward(*args)
     else:
         import ctypes

@@ -85,24 +85,29 @@ def test_shared_backward_matches_finite_differences():
         np.testing.assert_allclose(grad, numeric_grad(loss, arr), rtol=2e-6, atol=2e-6)
 
 
-def router_weights_closed_form(x, w, ids, scale):
-    p_all = 1.0 / (1.0 + np.exp(-(x @ w)))
+def router_weights_closed_form(x, w, ids, scale, score_func="sigmoid"):
+    z = x @ w
+    if score_func == "sigmoid":
+        p_all = 1.0 / (1.0 + np.exp(-z))
+    else:  # written independently of the oracle's helper: the definition, without the max shift
+        p_all = np.exp(z) / np.exp(z).sum(-1, keepdims=True)
     p = np.take_along_axis(p_all, ids, axis=-1)
     return scale * p / (p.sum(-1, keepdims=True) + 1e-20), p_all
 
 
+@pytest.mark.parametrize("score_func", ["sigmoid", "softmax"])
 @pytest.mark.parametrize("with_score_cotangent", [False, True])
-def test_router_backward_matches_finite_differences(with_score_cotangent):
+def test_router_backward_matches_finite_differences(with_score_cotangent, score_func):
     rng = np.random.default_rng(4)
     T, H, E, K, scale = 6, 5, 7, 3, 2.5
     x, w = rng.standard_normal((T, H)), rng.standard_normal((H, E)) * 0.7
     ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int64)  # the selection is held fixed
     d_weights = rng.standard_normal((T, K))
     d_scores = rng.standard_normal((T, E)) if with_score_cotangent else None
-    got = G.router_backward(x, w, ids, d_weights, d_scores, scale)
+    got = G.router_backward(x, w, ids, d_weights, d_scores, scale, score_func=score_func)
 
     def loss():
-        weights, scores = router_weights_closed_form(x, w, ids, scale)
+        weights, scores = router_weights_closed_form(x, w, ids, scale, score_func)
         extra = float(np.sum(scores * d_scores)) if with_score_cotangent else 0.0
         return float(np.sum(weights * d_weights)) + extra
 
@@ -110,7 +115,8 @@ def test_router_backward_matches_finite_differences(with_score_cotangent):
     np.testing.assert_allclose(got.d_w_router, numeric_grad(loss, w), rtol=2e-6, atol=2e-6)
 
 
-def test_layer_backward_matches_finite_differences():
+@pytest.mark.parametrize("score_func", ["sigmoid", "softmax"])
+def test_layer_backward_matches_finite_differences(score_func):
     rng = np.random.default_rng(5)
     T, H, E, K, I, Is, scale = 7, 4, 5, 2, 6, 3, 1.5
     x, w = rng.standard_normal((T, H)), rng.standard_normal((H, E)) * 0.7
@@ -122,12 +128,12 @@ def test_layer_backward_matches_finite_differences():
     dy, d_scores = rng.standard_normal((T, H)), rng.standard_normal((T, E))
 
     def layer():
-        weights, scores = router_weights_closed_form(x, w, ids, scale)
+        weights, scores = router_weights_closed_form(x, w, ids, scale, score_func)
         y = dense_experts(x, ids, weights, gate, up, down) + (silu(x @ shared[0]) * (x @ shared[1])) @ shared[2]
         return y, scores, weights
 
     weights0 = layer()[2]
-    got = G.moe_backward(x, w, gate, up, down, shared, ids, weights0, dy, d_scores, scale)
+    got = G.moe_backward(x, w, gate, up, down, shared, ids, weights0, dy, d_scores, scale, score_func=score_func)
 
     def loss():
         y, scores, _ = layer()

@@ -99,6 +99,50 @@ def test_router_invariants_random_bf16():
     np.testing.assert_allclose(r.weights.sum(-1), 2.5, rtol=2e-2)
 
 
+def test_softmax_scores_against_float64_closed_forms():
+    """The softmax score function is not a reference path (moe.py:133 is a sigmoid): it is pinned by what
+    the definition fixes."""
+    rng = np.random.default_rng(11)
+    for experts in (3, 5, 16, 64, 130, 256):
+        z = (rng.standard_normal((40, experts)) * 4.0).astype(np.float32)
+        z[0, :] = 1.25            # all equal: exactly uniform up to the rounding of one division
+        z[1, :] = -200.0
+        z[1, experts // 2] = 50.0  # one dominant logit: everything else is clamped at exp(-86)
+        s = O.softmax_f32(z)
+        z64 = z.astype(np.float64)
+        ref = np.exp(z64 - z64.max(-1, keepdims=True))
+        ref /= ref.sum(-1, keepdims=True)
+        big = ref > 1e-30
+        np.testing.assert_allclose(s[big], ref[big], rtol=3e-6)
+        assert np.all(s[~big] < 1e-30)
+        np.testing.assert_allclose(s.sum(-1), 1.0, rtol=1e-6)
+        np.testing.assert_allclose(s[0], 1.0 / experts, rtol=3e-7)
+        assert s[1, experts // 2] == 1.0
+        # order-preserving: a larger logit never gets a smaller score
+        order = np.argsort(z[2])
+        assert np.all(np.diff(s[2][order]) >= 0)
+    # adding a constant to a row that keeps the differences exact does not change anything
+    z = np.array([[0.5, -1.25, 3.0, 2.0]], np.float32)
+    assert np.array_equal(O.softmax_f32(z), O.softmax_f32(z + np.float32(8.0)))
+
+
+def test_softmax_router_selection_and_weights():
+    logits = np.array([[2.0, 0.0, -2.0, 1.0]], np.float32)
+    r = O.router_from_logits(logits, None, 2, 1.5, "f32", "softmax")
+    assert r.expert_ids.tolist() == [[0, 3]]
+    e = [math.exp(v) for v in (2.0, 0.0, -2.0, 1.0)]
+    s = [v / sum(e) for v in e]
+    np.testing.assert_allclose(r.scores[0], s, rtol=2e-6)
+    np.testing.assert_allclose(r.weights[0], [1.5 * s[0] / (s[0] + s[3]), 1.5 * s[3] / (s[0] + s[3])], rtol=2e-6)
+    # the bias enters the selection only, ties go to the lower index, as with the sigmoid
+    biased = O.router_from_logits(logits, np.array([0, 0, 5.0, 0], np.float32), 2, 1.0, "f32", "softmax")
+    assert biased.expert_ids.tolist() == [[2, 0]]
+    tied = O.router_from_logits(np.zeros((1, 6), np.float32), None, 3, 1.0, "f32", "softmax")
+    assert tied.expert_ids.tolist() == [[0, 1, 2]]
+    with pytest.raises(ValueError):
+        O.router_from_logits(logits, None, 2, 1.0, "f32", "tanh")
+
+
 def test_router_argument_errors():
     logits = np.zeros((2, 4), np.float32)
     with pytest.raises(ValueError):
