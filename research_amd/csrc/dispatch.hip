@@ -153,10 +153,10 @@ __global__ __launch_bounds__(kScanThreads) void dispatch_scan_kernel(int* __rest
 constexpr int kDirectMaxChunks = 256;
 
 // LDS of the rank pass: imp[E] of 8 bytes (kDirect && kStats), cursor[E], wavehist[kDispWaves][E],
-// and for kDirect tot[slots], pre[slots], wave_s[kDispWaves] with slots = max(E, kDispThreads)
+// and for kDirect tot[kDispThreads], pre[kDispThreads], wave_s[kDispWaves]
 inline size_t rank_smem_bytes(int E, bool direct, bool stats) {
   size_t n = (size_t)E * (1 + kDispWaves) * sizeof(int);
-  if (direct) n += ((size_t)2 * (E > kDispThreads ? E : kDispThreads) + kDispWaves) * sizeof(int);
+  if (direct) n += ((size_t)2 * kDispThreads + kDispWaves) * sizeof(int);
   if (direct && stats) n += (size_t)E * 8;
   return n;
 }
@@ -170,71 +170,54 @@ __device__ __forceinline__ void chunk_bases(const int* __restrict__ partial,
                                             int* cursor, int* tmp, unsigned long long* imp_s,
                                             int32_t* __restrict__ group_sizes, int32_t* __restrict__ offsets,
                                             float* __restrict__ expert_counts, float* __restrict__ importance) {
+  static_assert(JTMOE_MAX_EXPERTS <= kDispThreads, "one thread per expert in the scan over the experts");
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  const int slots = E > kDispThreads ? E : kDispThreads;
-  int* const tot_s = tmp;
-  int* const pre_s = tmp + slots;
-  int* const wave_s = pre_s + slots;
+  int* const tot_s = tmp;                  // [kDispThreads]
+  int* const pre_s = tmp + kDispThreads;   // [kDispThreads]
+  int* const wave_s = pre_s + kDispThreads;
   const bool first = blockIdx.x == 0;
-  if (kStats && first)
+  if (kStats && first) {
     for (int e = tid; e < E; e += kDispThreads) imp_s[e] = 0ull;
-  if (kStats && first) __syncthreads();
-  // G groups of E threads share out the chunks (chunk c goes to group c % G); with more experts than
-  // threads every thread takes several experts and all chunks
-  const int G = E <= kDispThreads ? kDispThreads / E : 1;
-  for (int e0 = 0; e0 < E; e0 += kDispThreads) {
-    int g = 0, e = e0 + tid;
-    if (E <= kDispThreads) {
-      g = tid / E;
-      e = tid - g * E;
-    }
-    if (g < G && e < E) {
-      int tot = 0, pre = 0;
-      unsigned long long acc = 0ull;
-      // 16 loads in flight at a time: the table is in the L2, what costs is the round trip
-      constexpr int kBatch = 16;
-      for (int c0 = g; c0 < nchunks; c0 += kBatch * G) {
-        int v[kBatch];
-        unsigned long long w[kBatch];
+    __syncthreads();
+  }
+  // G groups of E threads share out the chunks: chunk c goes to group c % G
+  const int G = kDispThreads / E;
+  const int g = tid / E, e = tid - g * E;
+  if (g < G) {
+    int tot = 0, pre = 0;
+    unsigned long long acc = 0ull;
+    // 16 loads in flight at a time: the table is in the L2, what costs is the round trip
+    constexpr int kBatch = 16;
+    for (int c0 = g; c0 < nchunks; c0 += kBatch * G) {
+      int v[kBatch];
+      unsigned long long w[kBatch];
 #pragma unroll
-        for (int j = 0; j < kBatch; ++j) {
-          const int c = c0 + j * G;
-          v[j] = c < nchunks ? partial[(size_t)c * E + e] : 0;
-          if (kStats && first) w[j] = c < nchunks ? partial_imp[(size_t)c * E + e] : 0ull;
-        }
-#pragma unroll
-        for (int j = 0; j < kBatch; ++j) {
-          const int c = c0 + j * G;
-          tot += v[j];
-          pre += c < (int)blockIdx.x ? v[j] : 0;
-          if (kStats && first) acc += w[j];
-        }
+      for (int j = 0; j < kBatch; ++j) {
+        const int c = c0 + j * G;
+        v[j] = c < nchunks ? partial[(size_t)c * E + e] : 0;
+        if (kStats && first) w[j] = c < nchunks ? partial_imp[(size_t)c * E + e] : 0ull;
       }
-      tot_s[g * E + e] = tot;
-      pre_s[g * E + e] = pre;
-      if (kStats && first) atomicAdd(&imp_s[e], acc);
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int c = c0 + j * G;
+        tot += v[j];
+        pre += c < (int)blockIdx.x ? v[j] : 0;
+        if (kStats && first) acc += w[j];
+      }
     }
-    if (E <= kDispThreads) break;
+    tot_s[tid] = tot;
+    pre_s[tid] = pre;
+    if (kStats && first) atomicAdd(&imp_s[e], acc);
   }
   __syncthreads();
-  // thread t owns the experts [t * per, t * per + per): their totals, then an exclusive scan over the threads
-  const int per = (E + kDispThreads - 1) / kDispThreads;  // <= 4
-  int tots[4], pres[4], mine = 0;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int e = tid * per + j;
-    int t = 0, q = 0;
-    if (j < per && e < E) {
-      for (int g = 0; g < G; ++g) {
-        t += tot_s[g * E + e];
-        q += pre_s[g * E + e];
-      }
+  // thread e owns expert e: its total over the groups, then an exclusive scan over the experts
+  int total = 0, before = 0;
+  if (tid < E)
+    for (int gg = 0; gg < G; ++gg) {
+      total += tot_s[gg * E + tid];
+      before += pre_s[gg * E + tid];
     }
-    tots[j] = t;
-    pres[j] = q;
-    mine += t;
-  }
-  int incl = mine;
+  int incl = total;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
     const int v = __shfl_up(incl, d);
@@ -242,22 +225,17 @@ __device__ __forceinline__ void chunk_bases(const int* __restrict__ partial,
   }
   if (lane == kWave - 1) wave_s[wave] = incl;
   __syncthreads();
-  int run = incl - mine;
-  for (int w = 0; w < wave; ++w) run += wave_s[w];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int e = tid * per + j;
-    if (j < per && e < E) {
-      cursor[e] = run + pres[j];
-      if (first) {
-        offsets[e] = run;
-        group_sizes[e] = tots[j];
-        if (kStats) {
-          expert_counts[e] = (float)tots[j];
-          importance[e] = (float)((double)imp_s[e] * (1.0 / 4294967296.0));
-        }
+  int start = incl - total;
+  for (int w = 0; w < wave; ++w) start += wave_s[w];
+  if (tid < E) {
+    cursor[tid] = start + before;
+    if (first) {
+      offsets[tid] = start;
+      group_sizes[tid] = total;
+      if (kStats) {
+        expert_counts[tid] = (float)total;
+        importance[tid] = (float)((double)imp_s[tid] * (1.0 / 4294967296.0));
       }
-      run += tots[j];
     }
   }
 }
