@@ -83,3 +83,37 @@ def test_layer_statistics_do_not_depend_on_what_the_buffers_held(gpu):
         assert torch.equal(layer.expert_counts, route.expert_counts), tokens
         assert torch.equal(layer.importance, route.importance), tokens
         assert float(layer.expert_counts.sum()) == tokens * K
+
+
+def test_layer_routing_outputs_on_seeded_random_shapes(gpu):
+    """Forty shapes drawn from a fixed seed (expert counts 1 ... 256 including odd ones, top-k up to 16,
+    batches from one token to a few thousand, hidden sizes the matrix-core router takes and others):
+    the layer call against the stand-alone entry points, bit for bit, for both score functions."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        experts = int(rng.choice([1, 2, 3, 5, 8, 16, 24, 32, 63, 64, 100, 128, 255, 256]))
+        top_k = int(rng.integers(1, min(experts, 16) + 1))
+        tokens = int(rng.choice([1, 2, 15, 16, 17, 63, 64, 65, 200, 256, 257, 600, 1030, 2500]))
+        hidden = int(rng.choice([8, 40, 64, 128, 192, 256]))
+        d_ff = int(rng.choice([8, 24, 64]))
+        dtype = "bf16" if rng.random() < 0.75 else "f32"
+        score_func = "softmax" if rng.random() < 0.3 else "sigmoid"
+        x = dev(rng.standard_normal((tokens, hidden)).astype(np.float32), gpu, dtype)
+        w_router = dev((rng.standard_normal((hidden, experts)) * 0.2).astype(np.float32), gpu, dtype)
+        bias = dev((rng.standard_normal(experts) * 0.01).astype(np.float32), gpu) if rng.random() < 0.5 else None
+        gate = dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, dtype)
+        up = dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, dtype)
+        down = dev((rng.standard_normal((experts, d_ff, hidden)) * 0.05).astype(np.float32), gpu, dtype)
+        tag = f"case {case}: T={tokens} H={hidden} E={experts} K={top_k} I={d_ff} {dtype} {score_func}"
+        print("[layer paths]", tag, flush=True)
+        layer = ops.moe_forward(x, w_router, bias, gate, up, down, top_k, 1.0, score_func=score_func)
+        route = ops.router(x, w_router, bias, top_k, 1.0, score_func=score_func)
+        plan = ops.dispatch(route.expert_ids, experts)
+        for name in ("expert_ids", "weights", "scores", "expert_counts", "importance"):
+            assert torch.equal(getattr(layer, name), getattr(route, name)), f"{tag}: {name}"
+        for name in ("group_sizes", "offsets", "source_order", "inverse"):
+            assert torch.equal(getattr(layer, name), getattr(plan, name)), f"{tag}: {name}"
+        d = O.dispatch(host(route.expert_ids), experts)
+        assert np.array_equal(host(plan.source_order), d.source_order), tag
+        assert np.array_equal(host(plan.group_sizes), d.group_sizes), tag
+        assert bool(torch.isfinite(layer.y.float()).all()), tag
