@@ -2,7 +2,9 @@
 // per-expert counts / importance of the router statistics.
 //
 // Follows SigmoidTopKRouter.__call__ (reference moe.py:131-147) and the two
-// vector outputs of _router_stats (moe.py:802-805).
+// vector outputs of _router_stats (moe.py:802-805).  The _sf entry points take the
+// score function as an attribute: the reference's sigmoid, or a softmax over the
+// experts (which the reference does not have) in front of the same selection.
 //
 // This file is compiled with floating-point contraction OFF and correctly
 // rounded fp32 division: everything after the logits is a fixed sequence of
