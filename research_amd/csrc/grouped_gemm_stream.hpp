@@ -316,6 +316,7 @@ __device__ __forceinline__ void stream_gemm_body(
     // LDS reads (two per MFMA) that were written before them
     // (`first`: the tile's first sub-step, which accumulates onto zero instead of clearing 128 registers)
     auto mfma_substep = [&](int cur_set, bool first = false) {
+      if (Cfg::OPT & 32) __builtin_amdgcn_s_setprio(1);
       f32x16_t zero;
 #pragma unroll
       for (int i = 0; i < 16; ++i) zero[i] = 0.0f;
@@ -330,6 +331,7 @@ __device__ __forceinline__ void stream_gemm_body(
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       }
+      if (Cfg::OPT & 32) __builtin_amdgcn_s_setprio(0);
     };
     // sub-steps 0 .. KK-2 of a step: fragments of the following sub-step are requested, then this one's MFMAs
     auto leading_substeps = [&](auto first_tag) {
@@ -354,6 +356,7 @@ __device__ __forceinline__ void stream_gemm_body(
         // (into the stage just released) and one fragment read of step j + 1 are issued
         const int ns = (cs + 1) & (NS - 1);
         constexpr int cur_set = (KK - 1) & 1;
+        if (Cfg::OPT & 32) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int g = 0; g < TM * TN; ++g) {
           acc[g / TN][g % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[cur_set][g % TN], af[cur_set][g / TN],
@@ -370,6 +373,7 @@ __device__ __forceinline__ void stream_gemm_body(
             bf[0][g - TM] = load_frag_b(ns, 0, g - TM);
           __builtin_amdgcn_sched_barrier(0);
         }
+        if (Cfg::OPT & 32) __builtin_amdgcn_s_setprio(0);
         cs = ns;
       };
       steady_step(std::true_type{});  // nk >= 2 NS: the steady part has at least NS steps

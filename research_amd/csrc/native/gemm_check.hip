@@ -11,6 +11,7 @@
 //                           with parts of its loop left out, and a fixed launch sequence for counter runs
 //   gemm_check time_stream_nt   the transposed-B form of the stream kernel against grouped_gemm_nt_kernel
 //   gemm_check time_ragged      the C3 launches on random against equal group sizes
+//   gemm_check time_prio        the stream kernel with and without raised wave priority around its MFMAs
 //   (a second argument "nocheck" skips the correctness cases)
 #include "grouped_gemm_bwd.hpp"
 #include "grouped_gemm_stream.hpp"
@@ -731,6 +732,17 @@ int main(int argc, char** argv) {
     }
     hipFree(A1);
     release(z); release(x);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_prio")) {
+    using Prio = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 32>;
+    Problem g = make(64, 131072, 2048, 1408, 4, false, 8, 1.0f);
+    g_stream = true;
+    for (int rep = 0; rep < 3; ++rep) {
+      timeit<GateUpStreamCfg>("gate/up stream", g, 20);
+      timeit<Prio>("gate/up stream, wave priority around the MFMAs", g, 20);
+    }
+    g_stream = false;
+    release(g);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_ragged")) {
     // What the ragged last tile of every group costs: the C3 launches on groups of random sizes
