@@ -295,6 +295,8 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
   __syncthreads();
 
   // selection: 4 lanes per token, each owning a contiguous quarter of the experts
+  // (sixteen lanes per token, where a workgroup has them to spare, measured no faster: a round costs
+  // its chain of dependent steps, not its compares)
   const int t = tid >> 2, q = tid & 3;
   const int eq = (E + 3) >> 2;
   const int e_begin = q * eq;
@@ -313,12 +315,14 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
   } else {
     select_from_lds(sm, row, e_begin, eq, E, row_ok, t, q, K);
   }
-  // renormalise (lane 0 of the token; it wrote top_* itself)
-  if (row_ok && q == 0) {
+  __syncthreads();  // the selection of a token was written by its lane 0 and is read by all its lanes
+  // renormalise: the lanes of a token share out its K slots; each adds up the denominator itself, in
+  // slot order
+  if (row_ok) {
     float denom = sm.top_score[t * K];
     for (int r = 1; r < K; ++r) denom = denom + sm.top_score[t * K + r];
     denom = denom + 1e-20f;
-    for (int r = 0; r < K; ++r) {
+    for (int r = q; r < K; r += 4) {
       const int e = sm.top_id[t * K + r];
       float w = sm.top_score[t * K + r] / denom;
       w = w * route_scale;
