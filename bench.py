@@ -109,8 +109,8 @@ def cpu_baseline(name: str, sample_tokens: int | None) -> dict:
         kind="port",
         sample=(f"all {sample_tokens} tokens of {name}" if whole else f"first {sample_tokens} tokens of {name}")
                + f" (seed-0 weights), NumPy oracle, {'emulated bf16' if cfg['dtype'] == 'bf16' else 'fp32'}, "
-                 (f"{calls} timed calls of {dt:.3f} s each" if calls > 1 else f"one timed call of {dt:.2f} s")
-                 + " after a 64-token warm-up call",
+               + (f"{calls} timed calls of {dt:.3f} s each" if calls > 1 else f"one timed call of {dt:.2f} s")
+               + " after a 64-token warm-up call",
     )
 
 
