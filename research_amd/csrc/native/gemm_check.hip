@@ -11,6 +11,7 @@
 //                           with parts of its loop left out, and a fixed launch sequence for counter runs
 //   gemm_check time_stream_nt   the transposed-B form of the stream kernel against grouped_gemm_nt_kernel
 //   gemm_check time_ragged      the C3 launches on random against equal group sizes
+//   gemm_check time_c2_down     the down projection with 256 x 256 against 256 x 128 tiles, caches warm and cold
 //   gemm_check time_prio        the stream kernel with and without raised wave priority around its MFMAs
 //   (a second argument "nocheck" skips the correctness cases)
 #include "grouped_gemm_bwd.hpp"
@@ -230,6 +231,38 @@ static void timeit(const char* name, Problem& p, int iters) {
   const double flops = 2.0 * p.rows * (double)p.K * p.N * (Cfg::kDual ? 2 : 1);
   printf("time %-36s rows=%d K=%d N=%d: %.3f ms  %.1f TFLOP/s  (%.1f%% of 2500)\n", name, p.rows, p.K, p.N, ms,
          flops / ms / 1e9, flops / ms / 1e9 / 25.0);
+  fflush(stdout);
+}
+
+// The same with the caches cold: between two timed launches a fill of 1 GiB goes through the L2s and
+// the memory-side cache, so that the operands come from HBM as they do inside a layer, where the
+// launch before has streamed other matrices.  Each launch is timed by its own pair of events.
+__global__ __launch_bounds__(256) void flush_fill_kernel(u32x4_t* out, size_t n) {
+  const u32x4_t v = {1u, 2u, 3u, 4u};
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) out[i] = v;
+}
+template <typename Cfg>
+static void timeit_cold(const char* name, Problem& p, int iters) {
+  static u32x4_t* junk = nullptr;
+  const size_t junk_vecs = (size_t)1 << 26;
+  if (junk == nullptr) CK(hipMalloc(&junk, junk_vecs * 16));
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
+  for (int i = 0; i < 20; ++i) launch<Cfg>(p, false);
+  double total = 0;
+  for (int i = 0; i < iters; ++i) {
+    flush_fill_kernel<<<4096, 256>>>(junk, junk_vecs);
+    CK(hipEventRecord(a));
+    launch<Cfg>(p, false);
+    CK(hipEventRecord(b)); CK(hipEventSynchronize(b));
+    float ms;
+    CK(hipEventElapsedTime(&ms, a, b));
+    total += ms;
+  }
+  const double ms = total / iters;
+  const double flops = 2.0 * p.rows * (double)p.K * p.N * (Cfg::kDual ? 2 : 1);
+  printf("time %-36s rows=%d K=%d N=%d: %.3f ms  %.1f TFLOP/s  (%.1f%% of 2500), caches cold\n", name, p.rows, p.K,
+         p.N, ms, flops / ms / 1e9, flops / ms / 1e9 / 25.0);
   fflush(stdout);
 }
 
@@ -732,6 +765,28 @@ int main(int argc, char** argv) {
     }
     hipFree(A1);
     release(z); release(x);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_c2_down")) {
+    // the down projection of the second configuration: 16 groups of about 1024 rows, K = 2816, N = 1024 --
+    // 288 tiles of 256 x 256 on 256 CUs (one full round and an eighth of a second one) against 576
+    // tiles of 256 x 128 -- which looks 8 % faster when the launch is repeated back to back (operands and result,
+    // 217 MB, stay in the memory-side cache) and is 15 % slower with the caches cold, as in a layer
+    using Half = DmaGemmCfg<256, 128, 64, 4, 2, false, 2, 16 + 64 + 128 + 32768>;
+    Problem d = make(16, 16384, 2816, 1024, 7, false, 0, 1.0f);
+    ok &= check<Half>("down, 256 x 128 tiles", d);
+    for (int rep = 0; rep < 3; ++rep) {
+      timeit<DownCfg>("C2 down, 256 x 256 tiles (library)", d, 20);
+      timeit<Half>("C2 down, 256 x 128 tiles", d, 20);
+      timeit_cold<DownCfg>("C2 down, 256 x 256 tiles (library)", d, 20);
+      timeit_cold<Half>("C2 down, 256 x 128 tiles", d, 20);
+    }
+    release(d);
+    Problem d3 = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
+    for (int rep = 0; rep < 2; ++rep) {
+      timeit<DownCfg>("C3 down, 256 x 256 tiles (library)", d3, 20);
+      timeit<Half>("C3 down, 256 x 128 tiles", d3, 20);
+    }
+    release(d3);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_prio")) {
     using Prio = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 32>;
