@@ -243,12 +243,14 @@ SplitPlan split_plan(int64_t rows, int64_t KA, int64_t N) {
   SplitPlan p{0, 0};
   const int64_t cus = persistent_grid_size();
   if (tiles > cus || rows < 2048) return p;
+  constexpr int64_t kStep = 64;  // the estimate counts in steps of 64 rows, whatever the kernel's k step
+  static_assert(kStep % Cfg::BK == 0, "a run is a whole number of k steps");
   const double reduce_steps = 0.84e-6 * (double)KA * (double)N * (Cfg::kDual ? 2.0 : 1.0);
   auto cost = [&](int64_t runs) {
-    const int64_t chunk = ((rows + runs - 1) / runs + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
+    const int64_t chunk = ((rows + runs - 1) / runs + kStep - 1) / kStep * kStep;
     const int64_t real_runs = (rows + chunk - 1) / chunk;
     const int64_t rounds = (tiles * real_runs + cus - 1) / cus;
-    return (double)rounds * (double)(chunk / Cfg::BK + 3) + (real_runs > 1 ? reduce_steps * (double)real_runs : 0.0);
+    return (double)rounds * (double)(chunk / kStep + 3) + (real_runs > 1 ? reduce_steps * (double)real_runs : 0.0);
   };
   const int64_t max_runs = std::min<int64_t>(64, rows / 256);
   int64_t best = 1;
@@ -261,7 +263,7 @@ SplitPlan split_plan(int64_t rows, int64_t KA, int64_t N) {
     }
   }
   if (best < 2 || best_cost > 0.9 * cost(1)) return p;
-  const int64_t chunk = ((rows + best - 1) / best + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
+  const int64_t chunk = ((rows + best - 1) / best + kStep - 1) / kStep * kStep;
   p.splits = (int)((rows + chunk - 1) / chunk);
   p.chunk = (int)chunk;
   return p;
@@ -316,12 +318,19 @@ int launch_gemm_tn(int dtype, const void* p, const void* d0, const void* d1, voi
   const bool fast = dtype == JTMOE_BF16 && KA % 8 == 0 && N % 8 == 0 && p_rows * KA < kOperandLimit &&
                     d_rows * N < kOperandLimit && aligned16(p) && aligned16(d0) && aligned16(c0) &&
                     (!dual || (aligned16(d1) && aligned16(c1)));
+  if (fast && (p_gather || d_gather)) {
+    if (dual)
+      return launch_tn_fast<WgradDualGatherCfg>(p, d0, d1, c0, c1, group_sizes, offsets, rows, KA, N, E, row_map,
+                                                row_div, p_gather, d_gather, gathered_rows, stream, split_ws);
+    return launch_tn_fast<WgradGatherCfg>(p, d0, nullptr, c0, nullptr, group_sizes, offsets, rows, KA, N, E, row_map,
+                                          row_div, p_gather, d_gather, gathered_rows, stream, split_ws);
+  }
   if (fast) {
     if (dual)
-      return launch_tn_fast<WgradDualCfg>(p, d0, d1, c0, c1, group_sizes, offsets, rows, KA, N, E, row_map, row_div,
-                                          p_gather, d_gather, gathered_rows, stream, split_ws);
-    return launch_tn_fast<WgradCfg>(p, d0, nullptr, c0, nullptr, group_sizes, offsets, rows, KA, N, E, row_map,
-                                    row_div, p_gather, d_gather, gathered_rows, stream, split_ws);
+      return launch_tn_fast<WgradDualCfg>(p, d0, d1, c0, c1, group_sizes, offsets, rows, KA, N, E, nullptr, 1, false,
+                                          false, 0, stream, split_ws);
+    return launch_tn_fast<WgradCfg>(p, d0, nullptr, c0, nullptr, group_sizes, offsets, rows, KA, N, E, nullptr, 1,
+                                    false, false, 0, stream, split_ws);
   }
   const int64_t mt = (KA + QB - 1) / QB, nt = (N + QB - 1) / QB;
   if (E * mt * nt >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm (tn): grid too large");

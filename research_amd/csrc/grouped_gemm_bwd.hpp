@@ -261,9 +261,12 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_nt_kernel(
 
 // ---------------------------------------------------------------------------------------------
 
-template <int BMO_, int BNO_, int WAVES_M_, int WAVES_N_, bool kDual_, int OPT_ = 16>
+// BK_ rows of the reduction per k step, NSTAGE_ operand stages in LDS: a step's loads are issued
+// NSTAGE_ - 1 steps before they are read.  More than two stages only for streamed operands (no row map).
+template <int BMO_, int BNO_, int WAVES_M_, int WAVES_N_, bool kDual_, int OPT_ = 16, int BK_ = 64, int NSTAGE_ = 2>
 struct TnGemmCfg {
-  static constexpr int BMO = BMO_, BNO = BNO_, BK = 64, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, OPT = OPT_;
+  static constexpr int BMO = BMO_, BNO = BNO_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, OPT = OPT_;
+  static constexpr int NSTAGE = NSTAGE_;
   static constexpr bool kDual = kDual_;
   static constexpr int BNE = kDual ? 2 * BNO : BNO;
   static constexpr int PSUB = BMO / 128, DSUB = BNE / 128;  // 128-column sub-tiles of the two operands
@@ -278,8 +281,10 @@ struct TnGemmCfg {
   static constexpr int SUB_LOADS = BK * 16 / NT;
   static constexpr int CS = WNO + 8;
   static constexpr size_t EPI_BYTES = (size_t)WAVES_M * WAVES_N * WM * CS * 2;
-  static constexpr size_t PIPE_BYTES = 2 * (size_t)STAGE_BYTES;
+  static constexpr int LOADS_PER_STAGE = (PSUB + DSUB) * SUB_LOADS;
+  static constexpr size_t PIPE_BYTES = NSTAGE * (size_t)STAGE_BYTES;
   static constexpr size_t SMEM_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
+  static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64), "two to four stages of 32 or 64 rows");
   static_assert(BMO % 128 == 0 && BNE % 128 == 0, "operand tiles are made of 128-column sub-tiles");
   static_assert((BK * 16) % NT == 0, "sub-tile must divide evenly over the threads");
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32x16 MFMAs");
@@ -326,7 +331,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
   int listed = -1;  // >= 0: this workgroup's pairs are s_list[0 .. listed)
   if (group_sizes) {
     constexpr int kPer = JTMOE_MAX_EXPERTS / 64;  // groups per lane, contiguous
-    constexpr int kFixedSteps = 3;                // look-up and epilogue of a pair, in k steps
+    constexpr int kFixedSteps = 3 * 64 / BK;      // look-up and epilogue of a pair, in k steps
     int w[kPer], local = 0, wmin = 0x7fffffff, wmax = 0;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
@@ -522,12 +527,17 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
       ids[j] = r < rows ? row_map[row0 + r] / row_div : -1;
     }
   };
+  // (row ids are fetched one step ahead of their loads: with more than two stages the row map is not used)
+  if (Cfg::NSTAGE > 2) {
+    p_gather = 0;
+    d_gather = 0;
+  }
   const bool any_gather = p_gather || d_gather;
 
   // Rows past the end of the group must contribute zeros: their offsets lie outside the
   // descriptor (which ends with the group, or is pushed there explicitly for gathered rows).
   auto issue = [&](int kt) {
-    const unsigned base = wave_lds + (kt & 1) * Cfg::STAGE_BYTES;
+    const unsigned base = wave_lds + (kt % Cfg::NSTAGE) * Cfg::STAGE_BYTES;
     int pv[Cfg::SUB_LOADS], dv[Cfg::SUB_LOADS];
 #pragma unroll
     for (int j = 0; j < Cfg::SUB_LOADS; ++j) {
@@ -537,19 +547,21 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
     }
     // LDS address = one scalar per stage + a compile-time offset per load (this kernel is short of
     // scalar registers)
-    static_assert(Cfg::PSUB <= 2 && Cfg::DSUB <= 2 && Cfg::SUB_LOADS == 2, "load list written out below");
+    static_assert(Cfg::PSUB <= 2 && Cfg::DSUB <= 2 && Cfg::SUB_LOADS <= 2, "load list written out below");
+    constexpr int L = Cfg::SUB_LOADS - 1;  // index of a sub-tile's second load (its first if there is one only)
     buffer_load_lds16_at<0>(p_rsrc, base, pv[0], 0);
-    buffer_load_lds16_at<NT * 16>(p_rsrc, base, pv[1], 0);
+    if (Cfg::SUB_LOADS == 2) buffer_load_lds16_at<NT * 16>(p_rsrc, base, pv[L], 0);
     if (Cfg::PSUB == 2) {
       buffer_load_lds16_at<Cfg::SUB_BYTES>(p_rsrc, base, pv[0] + 256, 0);
-      buffer_load_lds16_at<Cfg::SUB_BYTES + NT * 16>(p_rsrc, base, pv[1] + 256, 0);
+      if (Cfg::SUB_LOADS == 2) buffer_load_lds16_at<Cfg::SUB_BYTES + NT * 16>(p_rsrc, base, pv[L] + 256, 0);
     }
     buffer_load_lds16_at<Cfg::P_BYTES>(d_rsrc[0], base, dv[0], 0);
-    buffer_load_lds16_at<Cfg::P_BYTES + NT * 16>(d_rsrc[0], base, dv[1], 0);
+    if (Cfg::SUB_LOADS == 2) buffer_load_lds16_at<Cfg::P_BYTES + NT * 16>(d_rsrc[0], base, dv[L], 0);
     if (Cfg::DSUB == 2) {
       buffer_load_lds16_at<Cfg::P_BYTES + Cfg::SUB_BYTES>(d_rsrc[Cfg::DSUB - 1], base, dv[0] + (kDual ? 0 : 256), 0);
-      buffer_load_lds16_at<Cfg::P_BYTES + Cfg::SUB_BYTES + NT * 16>(d_rsrc[Cfg::DSUB - 1], base,
-                                                                  dv[1] + (kDual ? 0 : 256), 0);
+      if (Cfg::SUB_LOADS == 2)
+        buffer_load_lds16_at<Cfg::P_BYTES + Cfg::SUB_BYTES + NT * 16>(d_rsrc[Cfg::DSUB - 1], base,
+                                                                    dv[L] + (kDual ? 0 : 256), 0);
     }
   };
   // first loads of a tile (and, for gathered operands, the row ids they need)
@@ -623,25 +635,40 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
 
     // a wave whose block of the result lies wholly outside [KA, N] has nothing to add
     const bool wave_has_output = cur.m0 + wm * WM < KA && cur.n0 + wn * (kDual ? WN / 2 : WN) < N;
-    for (int kt = 0; kt < nk; ++kt) {
-      wait_vmcnt<0>();
-      __syncthreads();
-      if (kt + 1 < nk) {
-        issue(kt + 1);
-        if (any_gather && kt + 2 < nk) fetch_ids(kt + 2);
-      }
-      if (!wave_has_output) continue;
-      const unsigned char* st = smem_raw + (kt & 1) * Cfg::STAGE_BYTES;
-      bf16x8_t af[2][TM], bf[2][TN];
-      load_frags(st, 0, af[0], bf[0]);
+    auto mfma_substep = [&](const bf16x8_t* af, const bf16x8_t* bf) {
 #pragma unroll
-      for (int kk = 0; kk < BK / 16; ++kk) {
-        if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+      for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
-        for (int mi = 0; mi < TM; ++mi)
+        for (int jj = 0; jj < TN; ++jj)
+          acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bf[jj], acc[mi][jj], 0, 0, 0);
+    };
+    // Stage 0 of the tile is on its way (start_tile); the stages above it share their LDS with the
+    // epilogue's staging area, so their loads start behind the first barrier of the tile, by which
+    // every wave has stored its results: steps 1 .. NSTAGE - 1 all at once there, then one step per
+    // step, each NSTAGE - 1 steps ahead of its use.
+    int issued = 1;
+    {
+      for (int kt = 0; kt < nk; ++kt) {
+        // the stages younger than this step's stay in flight when the pipeline is full
+        if (Cfg::NSTAGE > 2 && issued - kt == Cfg::NSTAGE - 1)
+          wait_vmcnt<(Cfg::NSTAGE - 2) * Cfg::LOADS_PER_STAGE>();
+        else
+          wait_vmcnt<0>();
+        __syncthreads();
+        while (issued < nk && issued < kt + Cfg::NSTAGE) {
+          issue(issued);
+          ++issued;
+          if (any_gather && issued < nk) fetch_ids(issued);
+        }
+        if (!wave_has_output) continue;
+        const unsigned char* st = smem_raw + (kt % Cfg::NSTAGE) * Cfg::STAGE_BYTES;
+        bf16x8_t af[2][TM], bf[2][TN];
+        load_frags(st, 0, af[0], bf[0]);
 #pragma unroll
-          for (int jj = 0; jj < TN; ++jj)
-            acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
+        for (int kk = 0; kk < BK / 16; ++kk) {
+          if (kk + 1 < BK / 16) load_frags(st, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+          mfma_substep(af[kk & 1], bf[kk & 1]);
+        }
       }
     }
     __syncthreads();  // every wave is done reading the stage buffers (and, for an empty group, with
@@ -708,8 +735,15 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_tn_kernel(
 // Configurations the library launches.
 using DgradCfg = NtGemmCfg<256, 256, 2, 4, 16 + 64 + 32768>;   // data gradients: 256 x 256 tiles
 // narrow LDS blocks: the fastest layout when the operands are streamed (1.52 vs 1.60 ms for the
-// gate/up product of the C3 shape); the wide blocks pay off only when rows are gathered
-using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16 + 32768>;  // gate and up weight gradients share the x tile
-using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16 + 32768>;     // down weight gradient
+// gate/up product of the C3 shape); the wide blocks pay off only when rows are gathered.
+// Four stages of 32 rows against two of 64 (the same LDS): 1.39-1.43 against 1.47-1.49 ms for the gate/up
+// gradients of that shape, 0.73-0.75 against 0.76-0.77 ms for the down gradient; three stages measure
+// the same as four; moving a step's barrier in front of its last sub-step, which pays in the forward
+// kernel, costs 3-9 % here.
+using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16 + 32768, 32, 4>;  // gate and up weight gradients share the x tile
+using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16 + 32768, 32, 4>;     // down weight gradient
+// the same products with an operand fetched through a row map (row ids run one step ahead of their loads)
+using WgradDualGatherCfg = TnGemmCfg<256, 128, 4, 2, true, 16 + 32768>;
+using WgradGatherCfg = TnGemmCfg<256, 256, 2, 4, false, 16 + 32768>;
 
 }  // namespace jtmoe

@@ -68,6 +68,13 @@ __device__ __forceinline__ void buffer_load_lds16_nt(i32x4_t rsrc, unsigned lds_
                : "memory", "m0");
 }
 
+// s_waitcnt lgkmcnt(0) vmcnt(N), then the workgroup barrier.  The "memory" clobber keeps the
+// compiler from moving LDS accesses across it.
+template <int N>
+__device__ __forceinline__ void wait_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
 // fp32 -> bf16 by the hardware conversion (round to nearest even)
 __device__ __forceinline__ uint16_t bf16_bits_fast(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 __device__ __forceinline__ float bf16_round_fast(float f) { return (float)(__bf16)f; }

@@ -35,13 +35,6 @@ __device__ __forceinline__ void buffer_load_lds4(i32x4_t rsrc, unsigned lds_base
                : "memory", "m0");
 }
 
-// s_waitcnt lgkmcnt(0) vmcnt(N), then the workgroup barrier.  The "memory" clobber keeps the
-// compiler from moving LDS accesses across it.
-template <int N>
-__device__ __forceinline__ void wait_and_barrier() {
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
-}
-
 // two fp32 values -> their bf16 roundings packed in one dword (lo in the low half): one hardware conversion
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;

@@ -11,6 +11,7 @@
 //                           with parts of its loop left out, and a fixed launch sequence for counter runs
 //   gemm_check time_stream_nt   the transposed-B form of the stream kernel against grouped_gemm_nt_kernel
 //   gemm_check time_ragged      the C3 launches on random against equal group sizes
+//   gemm_check time_tn_stages   the weight-gradient kernel with two, three and four operand stages
 //   gemm_check time_c2_down     the down projection with 256 x 256 against 256 x 128 tiles, caches warm and cold
 //   gemm_check time_prio        the stream kernel with and without raised wave priority around its MFMAs
 //   (a second argument "nocheck" skips the correctness cases)
@@ -494,7 +495,7 @@ static void time_backward() {
     uint16_t *C0, *C1;
     CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
     time_launches("wgrad gate/up (gathered x^T @ dG, dU)", 4.0 * rows * H * I, 10,
-                  [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, true, false, false); });
+                  [&] { launch_tn<WgradDualGatherCfg>(p, D0, D1, C0, C1, true, false, false); });
     {  // the same product on a permuted copy of x: what the library runs
       uint16_t* Xp = random_bf16((size_t)rows * H, 36, 1.0f);
       Problem q = p;
@@ -522,7 +523,7 @@ static void time_backward() {
     Problem q = p;
     q.A = P;
     time_launches("wgrad down (act^T @ gathered dy)", 2.0 * rows * H * I, 10,
-                  [&] { launch_tn<WgradCfg>(q, D, nullptr, C0, nullptr, false, true, false); });
+                  [&] { launch_tn<WgradGatherCfg>(q, D, nullptr, C0, nullptr, false, true, false); });
     {
       uint16_t* dYp = random_bf16((size_t)rows * H, 37, 1.0f);
       time_launches("wgrad down (act^T @ packed dy)", 2.0 * rows * H * I, 10,
@@ -599,8 +600,8 @@ int main(int argc, char** argv) {
   {
     Problem p = make(5, 2400, 512, 384, 12, true, 3, 1.0f);
     ok &= check_nt<DgradCfg>("dgrad gather on load", p, 1);
-    ok &= check_tn<WgradDualCfg>("wgrad dual, transposed operand gathered", p, 1);
-    ok &= check_tn<WgradCfg>("wgrad, other operand gathered", p, 2);
+    ok &= check_tn<WgradDualGatherCfg>("wgrad dual, transposed operand gathered", p, 1);
+    ok &= check_tn<WgradGatherCfg>("wgrad, other operand gathered", p, 2);
     release(p);
   }
   {
@@ -654,8 +655,8 @@ int main(int argc, char** argv) {
     ok &= check_tn<WgradDualCfg>("wgrad dual many pairs per workgroup", u, 0);
     release(u);
     Problem v = make(70, 20000, 520, 264, 31, true, 3, 1.0f);  // the same with gathered operands and empty groups
-    ok &= check_tn<WgradDualCfg>("wgrad dual many pairs, transposed operand gathered", v, 1);
-    ok &= check_tn<WgradCfg>("wgrad many pairs, other operand gathered", v, 2);
+    ok &= check_tn<WgradDualGatherCfg>("wgrad dual many pairs, transposed operand gathered", v, 1);
+    ok &= check_tn<WgradGatherCfg>("wgrad many pairs, other operand gathered", v, 2);
     release(v);
     Problem w = make(256, 50000, 136, 264, 32, true, 0, 1.0f);  // the most groups, very unequal sizes
     ok &= check_tn<WgradCfg>("wgrad 256 unequal groups", w, 0);
@@ -910,6 +911,43 @@ int main(int argc, char** argv) {
       g_one_tile_per_workgroup = false;
       time_launches("wgrad gate/up, persistent (library)", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
       time_launches("wgrad down, persistent (library)", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+    }
+    hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
+    release(p); release(q);
+  }
+  if (ok && argc > 1 && !strcmp(argv[1], "time_tn_stages")) {
+    // the weight-gradient kernel with two stages of 64 rows, and three and four (the library's) of 32
+    using Dual64x2 = WgradDualGatherCfg;
+    using Dual32x3 = TnGemmCfg<256, 128, 4, 2, true, 16 + 32768, 32, 3>;
+    using Single64x2 = WgradGatherCfg;
+    using Single32x3 = TnGemmCfg<256, 256, 2, 4, false, 16 + 32768, 32, 3>;
+    {
+      Problem c = make(37, 50000, 512, 392, 41, false, 0, 1.0f);
+      ok &= check_tn<Dual32x3>("wgrad dual, 3 stages of 32", c, 0);
+      ok &= check_tn<Single32x3>("wgrad, 3 stages of 32", c, 0);
+      release(c);
+      Problem w = make(256, 60000, 256, 264, 43, true, 0, 1.0f);
+      ok &= check_tn<Dual32x3>("wgrad dual, 3 stages of 32, unequal groups", w, 0);
+      release(w);
+      Problem d = make(1, 5000, 512, 392, 47, false, 0, 1.0f);
+      ok &= check_tn<Single32x3>("wgrad, 3 stages of 32, dense", d, 0, true);
+      release(d);
+    }
+    const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
+    Problem p = make(E, rows, H, I, 21, false, 0, 1.0f);
+    uint16_t* D0 = random_bf16((size_t)rows * I, 31, 1.0f);
+    uint16_t* D1 = random_bf16((size_t)rows * I, 32, 1.0f);
+    uint16_t *C0, *C1;
+    CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
+    Problem q = make(E, rows, I, H, 23, false, 0, 1.0f);
+    uint16_t* dYp = random_bf16((size_t)rows * H, 37, 1.0f);
+    for (int rep = 0; ok && rep < 3; ++rep) {
+      time_launches("wgrad gate/up, 2 stages of 64", 4.0 * rows * H * I, 10, [&] { launch_tn<Dual64x2>(p, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad gate/up, 3 stages of 32", 4.0 * rows * H * I, 10, [&] { launch_tn<Dual32x3>(p, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad gate/up, 4 stages of 32 (library)", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad down, 2 stages of 64", 2.0 * rows * H * I, 10, [&] { launch_tn<Single64x2>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+      time_launches("wgrad down, 3 stages of 32", 2.0 * rows * H * I, 10, [&] { launch_tn<Single32x3>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+      time_launches("wgrad down, 4 stages of 32 (library)", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
     }
     hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
     release(p); release(q);
