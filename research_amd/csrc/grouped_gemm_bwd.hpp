@@ -739,7 +739,7 @@ using DgradCfg = NtGemmCfg<256, 256, 2, 4, 16 + 64 + 32768>;   // data gradients
 // Four stages of 32 rows against two of 64 (the same LDS): 1.39-1.43 against 1.47-1.49 ms for the gate/up
 // gradients of that shape, 0.73-0.75 against 0.76-0.77 ms for the down gradient; three stages measure
 // the same as four; moving a step's barrier in front of its last sub-step, which pays in the forward
-// kernel, costs 3-9 % here.
+// kernel, costs 3-9 % here, and asking the scheduler to put two transposing reads behind every MFMA 2-4 %.
 using WgradDualCfg = TnGemmCfg<256, 128, 4, 2, true, 16 + 32768, 32, 4>;  // gate and up weight gradients share the x tile
 using WgradCfg = TnGemmCfg<256, 256, 2, 4, false, 16 + 32768, 32, 4>;     // down weight gradient
 // the same products with an operand fetched through a row map (row ids run one step ahead of their loads)
