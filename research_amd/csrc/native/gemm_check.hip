@@ -662,6 +662,10 @@ int main(int argc, char** argv) {
     ok &= check_tn<WgradCfg>("wgrad 256 unequal groups", w, 0);
     ok &= check_tn<WgradDualCfg>("wgrad dual 256 unequal groups", w, 0);
     release(w);
+    Problem tiny = make(250, 7500, 256, 264, 49, false, 0, 1.0f);  // groups of about 30 rows: fewer k steps than stages
+    ok &= check_tn<WgradCfg>("wgrad tiny groups", tiny, 0);
+    ok &= check_tn<WgradDualCfg>("wgrad dual tiny groups", tiny, 0);
+    release(tiny);
   }
   {
     // the stream kernel: 32-deep steps with four stages, and 64-deep steps with two
@@ -949,6 +953,17 @@ int main(int argc, char** argv) {
       time_launches("wgrad down, 3 stages of 32", 2.0 * rows * H * I, 10, [&] { launch_tn<Single32x3>(q, dYp, nullptr, C0, nullptr, false, false, false); });
       time_launches("wgrad down, 4 stages of 32 (library)", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
     }
+    // what stands between the pairs of a workgroup: the same rows in half as many groups twice as
+    // long (half the pairs, the same matrix work)
+    Problem p2 = make(E / 2, rows, H, I, 21, false, 0, 1.0f);
+    Problem q2 = make(E / 2, rows, I, H, 23, false, 0, 1.0f);
+    for (int rep = 0; ok && rep < 2; ++rep) {
+      time_launches("wgrad gate/up, 64 groups", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad gate/up, 32 groups", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p2, D0, D1, C0, C1, false, false, false); });
+      time_launches("wgrad down, 64 groups", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
+      time_launches("wgrad down, 32 groups", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q2, dYp, nullptr, C0, nullptr, false, false, false); });
+    }
+    release(p2); release(q2);
     hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
     release(p); release(q);
   }
