@@ -11,6 +11,8 @@
 //                           with parts of its loop left out, and a fixed launch sequence for counter runs
 //   gemm_check time_stream_nt   the transposed-B form of the stream kernel against grouped_gemm_nt_kernel
 //   gemm_check time_ragged      the C3 launches on random against equal group sizes
+//   gemm_check time_decode      the decode-shape launches (64 groups of about 8 rows), also with the head of
+//                               every expert matrix read into the memory-side cache beforehand
 //   gemm_check time_tn_stages   the weight-gradient kernel with two, three and four operand stages
 //   gemm_check time_c2_down     the down projection with 256 x 256 against 256 x 128 tiles, caches warm and cold
 //   gemm_check time_prio        the stream kernel with and without raised wave priority around its MFMAs
@@ -536,9 +538,55 @@ static void time_backward() {
 }
 
 // decode-sized batch: 8 rows per group, bound by streaming the expert matrices
+// Reads the first `rows` rows of every expert's [K, N] matrix (both matrices of a dual launch) and
+// throws the data away: what is left behind is the data in the memory-side cache.
+__global__ __launch_bounds__(1024) void touch_rows_kernel(const u32x4_t* b0, const u32x4_t* b1, int E, size_t matrix_vecs,
+                                                          size_t head_vecs, unsigned* sink) {
+  const size_t total = (size_t)E * 2 * head_vecs;
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  for (size_t i = (size_t)blockIdx.x * 1024 + threadIdx.x; i < total; i += (size_t)gridDim.x * 1024) {
+    const size_t region = i / head_vecs, within = i - region * head_vecs;
+    const u32x4_t* base = (region & 1) ? b1 : b0;
+    const u32x4_t v = base[(region >> 1) * matrix_vecs + within];
+    acc[0] ^= v[0]; acc[1] ^= v[1]; acc[2] ^= v[2]; acc[3] ^= v[3];
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) *sink = 1;  // keeps the loads alive
+}
+
+// The decode-shape gate/up launch with the caches cold (a 1 GiB fill before every launch), and with the
+// first `head_rows` rows of every expert matrix read once between the fill and the launch.
+static void time_decode_prefetch(Problem& g, int head_rows, int iters) {
+  static u32x4_t* junk = nullptr;
+  static unsigned* sink = nullptr;
+  const size_t junk_vecs = (size_t)1 << 26;
+  if (junk == nullptr) { CK(hipMalloc(&junk, junk_vecs * 16)); CK(hipMalloc(&sink, 4)); }
+  hipEvent_t a, b, c;
+  CK(hipEventCreate(&a)); CK(hipEventCreate(&b)); CK(hipEventCreate(&c));
+  const size_t matrix_vecs = (size_t)g.K * g.N * 2 / 16, head_vecs = (size_t)head_rows * g.N * 2 / 16;
+  double touch_ms = 0, gemm_ms = 0;
+  for (int i = 0; i < iters + 3; ++i) {
+    flush_fill_kernel<<<4096, 256>>>(junk, junk_vecs);
+    CK(hipEventRecord(a));
+    if (head_rows > 0)
+      touch_rows_kernel<<<255, 1024>>>(reinterpret_cast<const u32x4_t*>(g.B0), reinterpret_cast<const u32x4_t*>(g.B1),
+                                       g.E, matrix_vecs, head_vecs, sink);
+    CK(hipEventRecord(b));
+    launch<GateUpTinyCfg>(g, false);
+    CK(hipEventRecord(c)); CK(hipEventSynchronize(c));
+    float t0, t1;
+    CK(hipEventElapsedTime(&t0, a, b)); CK(hipEventElapsedTime(&t1, b, c));
+    if (i >= 3) { touch_ms += t0; gemm_ms += t1; }
+  }
+  printf("time decode gate/up, caches cold, first %4d rows of each matrix touched before (%.1f MB): touch %.1f us, launch %.1f us\n",
+         head_rows, (double)g.E * 2 * head_vecs * 16 / 1e6, touch_ms / iters * 1e3, gemm_ms / iters * 1e3);
+  fflush(stdout);
+}
+
 static void time_decode() {
   Problem g = make(64, 512, 2048, 1408, 8, false, 0, 1.0f);
   Problem d = make(64, 512, 1408, 2048, 9, false, 0, 1.0f);
+  for (int rep = 0; rep < 2; ++rep)
+    for (int head : {0, 128, 256, 384, 512, 2048}) time_decode_prefetch(g, head, 20);
   timeit<GateUpCfg>("gate/up 64 groups, 256-row tiles", g, 20);
   timeit<DownCfg>("down 64 groups, 256-row tiles", d, 20);
   for (int rep = 0; rep < 3; ++rep) {
