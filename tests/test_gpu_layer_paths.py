@@ -89,8 +89,12 @@ def test_layer_routing_outputs_on_seeded_random_shapes(gpu):
     """Forty shapes drawn from a fixed seed (expert counts 1 ... 256 including odd ones, top-k up to 16,
     batches from one token to a few thousand, hidden sizes the matrix-core router takes and others):
     the layer call against the stand-alone entry points, bit for bit, for both score functions."""
-    rng = np.random.default_rng(2024)
-    for case in range(40):
+    check_random_layer_shapes(gpu, seed=2024, cases=40)
+
+
+def check_random_layer_shapes(gpu, seed: int, cases: int) -> None:
+    rng = np.random.default_rng(seed)
+    for case in range(cases):
         experts = int(rng.choice([1, 2, 3, 5, 8, 16, 24, 32, 63, 64, 100, 128, 255, 256]))
         top_k = int(rng.integers(1, min(experts, 16) + 1))
         tokens = int(rng.choice([1, 2, 15, 16, 17, 63, 64, 65, 200, 256, 257, 600, 1030, 2500]))

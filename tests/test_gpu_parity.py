@@ -22,6 +22,13 @@ BF16_MAX_REL = 2e-2  # max|y-ref| / max|ref|
 F32_TOL = dict(rtol=2e-5, atol=2e-5)
 
 
+def f32_tol(ref: np.ndarray) -> dict:
+    """fp32 bar for sums of hundreds of terms: the kernels add in k order, NumPy in blocks, so an
+    element that cancels to near zero differs by a few ulp of the *terms*; the absolute part of the
+    bar therefore follows the scale of the result."""
+    return dict(rtol=2e-5, atol=2e-5 * max(1.0, float(np.abs(ref).max(initial=0.0))))
+
+
 def dev(a: np.ndarray, gpu, dtype: str | None = None) -> torch.Tensor:
     t = torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
     if dtype == "bf16":
@@ -247,8 +254,8 @@ def test_grouped_swiglu_matches_oracle(gpu, tokens, hidden, experts, top_k, inte
         assert report(tag + " act", host(act), want_act) <= BF16_MAX_REL
         assert report(tag + " y", host(got), want) <= BF16_MAX_REL
     else:
-        np.testing.assert_allclose(host(act), want_act, **F32_TOL)
-        np.testing.assert_allclose(host(got), want, **F32_TOL)
+        np.testing.assert_allclose(host(act), want_act, **f32_tol(want_act))
+        np.testing.assert_allclose(host(got), want, **f32_tol(want))
 
 
 def test_grouped_swiglu_empty_groups_and_single_expert(gpu):
