@@ -834,6 +834,23 @@ int main(int argc, char** argv) {
       timeit_cold<Half>("C2 down, 256 x 128 tiles", d, 20);
     }
     release(d);
+    // the gate/up launch of the same configuration (gathered rows, K = 1024, N = 2816: 72 x 22 tiles of
+    // 256 x 128 + 128, 6.2 per CU) with the stream kernel's workgroups holding 4 tiles (library), 3, 2, 1,
+    // or one workgroup per CU walking its share (0)
+    {
+      Problem g2 = make(16, 16384, 1024, 2816, 6, false, 2, 1.0f);
+      g_stream = true;
+      for (int rep = 0; rep < 3; ++rep)
+        for (int chunk : {-1, 0, 1, 2, 3}) {
+          g_chunk = chunk;
+          char name[64];
+          snprintf(name, sizeof name, "C2 gate/up stream, %d tiles per workgroup", chunk < 0 ? 4 : chunk);
+          timeit_cold<GateUpStreamCfg>(name, g2, 20);
+        }
+      g_chunk = -1;
+      g_stream = false;
+      release(g2);
+    }
     Problem d3 = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
     for (int rep = 0; rep < 2; ++rep) {
       timeit<DownCfg>("C3 down, 256 x 256 tiles (library)", d3, 20);
