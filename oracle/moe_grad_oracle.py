@@ -35,6 +35,11 @@ Parity status (exercised in ``tests/test_oracle_grad.py``):
   three closed forms above with the selection held fixed.
 * sequence_balance_loss_backward: pinned by finite differences of the float64 closed
   form of the loss with the counts held fixed.
+* route_weight_grad_rounded: the same inner product as experts_backward's d_weights with the
+  four bf16 roundings a bf16 implementation makes on the way (the two products, the
+  activation, dy Wd^T); pinned against experts_backward by the first-order error bound that
+  those roundings allow (returned beside the value) and, with rounding switched off, by
+  equality with experts_backward.
 """
 
 from __future__ import annotations
@@ -89,6 +94,44 @@ def experts_backward(x, expert_ids, weights, gate, up, down, dy) -> ExpertsGrad:
         d_up[e] = xe.T @ du
         np.add.at(dx, t_idx, dg @ gate[e].T + du @ up[e].T)
     return ExpertsGrad(dx, d_weights, d_gate, d_up, d_down)
+
+
+def _bf16(a):
+    """float64 -> nearest bf16 (ties to even), returned as float64."""
+    b = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    b = ((b + 0x7FFF + ((b >> 16) & 1)) >> 16) << 16
+    return b.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
+def route_weight_grad_rounded(x, expert_ids, gate, up, down, dy, rounded=True):
+    """d_weights[t,s] = <dy[t], y_e(x[t])> evaluated as <Z, h> with Z = dy[t] Wd[e]^T and
+    h = silu(g) u, g = x[t] Wg[e], u = x[t] Wu[e] (the same number: both are dy^T Wd^T h), where a
+    bf16 implementation rounds g, u, h and Z to bf16 before the inner product and the result after it.
+
+    Returns (value, budget), both [T,K].  budget[t,s] = 2^-9 * (sum_i |Z_i h_i| (3 + kappa_i) + |value|)
+    with kappa = |d ln silu(g) / d ln g| = |1 + g (1 - sigmoid(g))|: the first-order bound on
+    |value - exact| from one relative rounding of 2^-9 on each of Z, u, h (factor 1 each) and g
+    (factor kappa), plus the rounding of the result.  With cancellation in the sum the exact value can
+    be far smaller than sum_i |Z_i h_i|, which is why a bound relative to the value itself (or, for a
+    tensor of one element, to the tensor's maximum) does not hold for this quantity.
+    """
+    x, gate, up, down, dy = (_f64(a) for a in (x, gate, up, down, dy))
+    ids = np.asarray(expert_ids)
+    rnd = _bf16 if rounded else (lambda a: a)
+    value = np.zeros(ids.shape)
+    budget = np.zeros(ids.shape)
+    for e in range(gate.shape[0]):
+        t_idx, s_idx = np.nonzero(ids == e)
+        if t_idx.size == 0:
+            continue
+        g, u = rnd(x[t_idx] @ gate[e]), rnd(x[t_idx] @ up[e])
+        sig = _sigmoid(g)
+        h = rnd(g * sig * u)
+        z = rnd(dy[t_idx] @ down[e].T)
+        value[t_idx, s_idx] = rnd(np.sum(z * h, axis=-1))
+        kappa = np.abs(1.0 + g * (1.0 - sig))
+        budget[t_idx, s_idx] = 2.0**-9 * (np.sum(np.abs(z * h) * (3.0 + kappa), axis=-1) + np.abs(value[t_idx, s_idx]))
+    return value, budget
 
 
 @dataclass

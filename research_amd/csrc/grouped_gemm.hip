@@ -229,11 +229,13 @@ int launch_stream(const void* a, const void* b0, const void* b1, void* c, const 
   return JTMOE_OK;
 }
 
-// what the stream kernel needs beyond fast_ok: enough k steps to fill its pipeline, a result below
-// 2^31 bytes (32-bit store offsets) and, with a row map, fewer than 2^27 rows and a divisor of at most 32
+// what the stream kernel needs beyond fast_ok: enough k steps to fill its pipeline, a result of at most
+// 0x7ffe0000 bytes (32-bit store offsets; the kernel drops a store by giving it the offset 0x7fff0000,
+// which must lie past the end of every admitted result) and, with a row map, fewer than 2^27 rows and a
+// divisor of at most 32
 template <typename Cfg>
 inline bool stream_ok(int64_t rows, int64_t Kdim, int64_t N, const int32_t* row_map, int row_div) {
-  return Kdim % Cfg::BK == 0 && Kdim / Cfg::BK >= 2 * Cfg::NSTAGE && rows * N * 2 < ((int64_t)1 << 31) &&
+  return Kdim % Cfg::BK == 0 && Kdim / Cfg::BK >= 2 * Cfg::NSTAGE && rows * N * 2 <= (int64_t)0x7ffe0000 &&
          (row_map == nullptr || (rows < ((int64_t)1 << 27) && row_div >= 1 && row_div <= 32));
 }
 

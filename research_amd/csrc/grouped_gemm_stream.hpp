@@ -16,7 +16,7 @@
 //     row map of the next tile arrives by LDS-DMA as well, group sizes and offsets are read from a copy
 //     in LDS), so the compiler never inserts a wait that drains the operand loads.
 //
-// Requirements: those of grouped_gemm_dma.hpp, and K / BK >= 2 * NSTAGE, a result of fewer than 2^31
+// Requirements: those of grouped_gemm_dma.hpp, and K / BK >= 2 * NSTAGE, a result of at most 0x7ffe0000
 // bytes, with a row map fewer than 2^27 rows and row_div <= 32; launch with a multiple of 8 workgroups
 // (persistent schedule).
 #pragma once
@@ -280,7 +280,8 @@ __device__ __forceinline__ void stream_gemm_body(
   if (cur.rows <= 0) return;
   Plan pl;
   plan_tile(pl, cur);
-  if (gather) plan_rows(pl, cur, [&](int r) { return row_map[cur.row0 + r]; });
+  // (a partial tile's rows past the group end are not read: the map may end with the group)
+  if (gather) plan_rows(pl, cur, [&](int r) { return r < cur.rows ? row_map[cur.row0 + r] : 0; });
 #pragma unroll
   for (int s = 0; s < NS; ++s) issue(pl, s, s);
   f32x16_t acc[TM][TN];
@@ -423,7 +424,8 @@ __device__ __forceinline__ void stream_gemm_body(
     // stores 16 contiguous bytes; no LDS staging, no barrier.
     // Stores go through a buffer descriptor of the whole result: one 32-bit offset per row, the
     // column of each store as an immediate, and rows past the end of the group (or columns past N)
-    // get an offset outside the buffer, which drops the store.
+    // get the offset 0x7fff0000, which lies outside every result the host admits (at most 0x7ffe0000
+    // bytes), so the hardware drops the store.
     // (the lane id is taken afresh so that nothing of the epilogue's addressing is kept in registers
     // through the k loops, where every register is spoken for)
     int lane_e;

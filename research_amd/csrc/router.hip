@@ -385,12 +385,27 @@ __global__ __launch_bounds__(256) void router_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// bf16 projection on the matrix cores.  One workgroup = 64 tokens = 4 waves of 16
-// tokens; each wave owns all E columns of its tokens (NB = E/16 accumulator tiles of
-// v_mfma_f32_16x16x32_bf16).  x is read straight from HBM into MFMA operand
-// registers (each lane 32 contiguous bytes per 64-wide k chunk, whole 128-byte
-// lines per token row); the router matrix [H,E] is staged chunk by chunk through
-// LDS as it is stored and read with the transposing ds_read_b64_tr_b16.
+// bf16 projection on the matrix cores.
+//
+// ONE summation order for every batch size.  A token's logits must not depend on how many tokens
+// share its call (a decode step of 64 tokens and a prefill of 16 384 have to route a row the same
+// way), although small batches want the k range shared out over many workgroups and large ones want
+// it walked by one.  All the matrix-core kernels below therefore add up a logit in this order:
+//   * H is cut into slices of router_slice_rows(H) consecutive k rows (eight slices, or as many
+//     128-row chunks as there are, when H is a multiple of 128; one slice otherwise);
+//   * inside a slice, v_mfma_f32_16x16x32_bf16 instructions are chained in k order, the first onto a
+//     zero accumulator, instruction n of the slice taking k = 32 n + 8 g + j at element j of lane
+//     group g (g = lane / 16) of both operands;
+//   * the slice sums are added in slice order, starting from the first slice's sum, and the total is
+//     rounded to bf16 (the projection's output dtype).
+// The large-batch kernel walks the slices one after the other with a second set of accumulators; the
+// small-batch kernels compute them in different workgroups and add them up afterwards.
+//
+// Large batches: one workgroup = 64 tokens = 4 waves of 16 tokens; each wave owns all E columns of
+// its tokens (NB = E/16 accumulator tiles).  x is read straight from HBM into MFMA operand registers
+// (each lane two 16-byte pieces per 64-wide k chunk, the four lane groups of a token together whole
+// 128-byte lines per token row); the router matrix [H,E] is staged chunk by chunk through LDS as it
+// is stored and read with the transposing ds_read_b64_tr_b16.
 // Requires H % 64 == 0 and E in {16, 32, 64, 128, 256}.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -400,6 +415,15 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 constexpr int kBufferFlags = 0x00020000;
 constexpr int kRouterKC = 64;  // k rows of the router matrix per LDS stage
+constexpr int kSplitKC = 128;  // k rows per LDS stage of the small-batch kernels; the unit the slices are cut in
+constexpr int kPartialMaxSlices = 8;
+
+// k rows per slice of the summation order (see above); a function of H only
+__host__ __device__ inline int router_slice_rows(int H) {
+  if (H % kSplitKC != 0) return H;
+  const int chunks = H / kSplitKC;
+  return (chunks + kPartialMaxSlices - 1) / kPartialMaxSlices * kSplitKC;
+}
 
 __host__ __device__ inline int router_w_stride(int E) { return E + 32; }  // elements; +64 B between k rows
 __host__ __device__ inline size_t router_mfma_smem_bytes(int E, int K, int tokens_per_wg) {
@@ -414,6 +438,7 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
     int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
     float* __restrict__ scores, float* __restrict__ logits_out, void* ws, int score_func) {
   constexpr int kRouterTokens = 16 * NW, kRouterThreads = 64 * NW;
+  const int slice_chunks = router_slice_rows(H) / kRouterKC;  // 64-row chunks per slice
   constexpr int E = NB * 16;
   constexpr int WS = E + 32;                      // LDS row stride of the staged matrix (elements)
   constexpr int W_CHUNKS = kRouterKC * E / 8;     // 16-byte chunks per stage
@@ -426,10 +451,10 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
   const int t0 = blockIdx.x * kRouterTokens;
   const int nrows = min(kRouterTokens, tokens - t0);
 
-  // x: lane (m = lane%16, kg = lane/16) holds k = chunk*64 + kg*16 + [0,16) of token t0 + wave*16 + m
+  // x: lane (m = lane%16, g = lane/16) holds k = chunk*64 + s*32 + g*8 + [0,8), s = 0, 1, of token t0 + wave*16 + m
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(x + (size_t)t0 * H), 0, nrows * H * 2, kBufferFlags);
-  const int x_voff = ((wave * 16 + (lane & 15)) * H + (lane >> 4) * 16) * 2;
+  const int x_voff = ((wave * 16 + (lane & 15)) * H + (lane >> 4) * 8) * 2;
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(w), 0, H * E * 2, kBufferFlags);
 
@@ -445,11 +470,11 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
   constexpr int UNROLL = D;  // a multiple of D and of the two LDS stages
   static_assert(D % 2 == 0, "the unrolled body alternates between the two LDS stages");
   u32x4_t a_ring[D][2], w_ring[D][CW];
-  f32x4_t acc[NB];
+  f32x4_t acc[NB], total[NB];  // the current slice's sum, and the sum of the slices before it
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[nb][i] = 0.0f;
+    for (int i = 0; i < 4; ++i) acc[nb][i] = total[nb][i] = 0.0f;
 
 #define JT_LOAD_W(slot, k0)                                                                  \
   _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                           \
@@ -468,12 +493,13 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
 #define JT_LOAD_X(slot, k0)                                                                  \
   {                                                                                          \
     a_ring[slot][0] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff, (k0)*2, 0);      \
-    a_ring[slot][1] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff + 16, (k0)*2, 0); \
+    a_ring[slot][1] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff + 64, (k0)*2, 0); \
   }
 
-  // transposing read of this lane: 16-lane group kg = lane/16 reads rows kg*16 + 8*s + 4*h + i/4
-  const int w_lane = ((lane >> 4) * 16 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
+  // transposing read of this lane: 16-lane group g = lane/16 reads rows 32*s + 8*g + 4*h + i/4
+  const int w_lane = ((lane >> 4) * 8 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
   const int nchunks = H / kRouterKC;
+  int in_slice = 0;  // chunks of the current slice done
 #pragma unroll
   for (int d = 0; d < D; ++d)
     if (d < nchunks) {
@@ -489,52 +515,39 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
       if (kc < nchunks) {  // uniform over the workgroup
         constexpr int kStages = 2;
         const int stage = j % kStages, slot = j % D, next_slot = (j + 1) % D;
-        if (D == 1 && kc + 1 < nchunks) {
-          // one slot: it is refilled before the MFMAs, which copy the operand out first
-          const u32x4_t a0 = a_ring[0][0], a1 = a_ring[0][1];
-          JT_LOAD_W(0, (kc + 1) * kRouterKC);
-          JT_LOAD_X(0, (kc + 1) * kRouterKC);
-          const uint16_t* wbase = Ws + stage * kRouterKC * WS + w_lane;
+        static_assert(D > 1, "a slot is refilled after the MFMAs that read it");
+        const uint16_t* wbase = Ws + stage * kRouterKC * WS + w_lane;
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, s ? a1 : a0);
+        for (int s = 0; s < 2; ++s) {
+          const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_ring[slot][s]);
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-              const uint16_t* p = wbase + s * 8 * WS + nb * 16;
-              const s16x4_t lo =
-                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
-              const s16x4_t hi =
-                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
-              const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-              acc[nb] =
-                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
-            }
+          for (int nb = 0; nb < NB; ++nb) {
+            const uint16_t* p = wbase + s * 32 * WS + nb * 16;
+            const s16x4_t lo =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+            const s16x4_t hi =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
+            const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            acc[nb] =
+                __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
           }
-          JT_STORE_W(0, stage ^ 1);
-        } else {
-          const uint16_t* wbase = Ws + stage * kRouterKC * WS + w_lane;
+        }
+        if (kc + 1 < nchunks) JT_STORE_W(next_slot, stage ^ 1);
+        if (kc + D < nchunks) {
+          JT_LOAD_W(slot, (kc + D) * kRouterKC);
+          JT_LOAD_X(slot, (kc + D) * kRouterKC);
+        }
+        // end of a slice (uniform; the last slice may be shorter): its sum joins the total, in slice order
+        if (++in_slice == slice_chunks || kc + 1 == nchunks) {
+          const bool first = kc < slice_chunks;
+          in_slice = 0;
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_ring[slot][s]);
+          for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-              const uint16_t* p = wbase + s * 8 * WS + nb * 16;
-              const s16x4_t lo =
-                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
-              const s16x4_t hi =
-                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
-              const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-              acc[nb] =
-                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
+            for (int i = 0; i < 4; ++i) {
+              total[nb][i] = first ? acc[nb][i] : total[nb][i] + acc[nb][i];
+              acc[nb][i] = 0.0f;
             }
-          }
-          if (D > 1) {
-            if (kc + 1 < nchunks) JT_STORE_W(next_slot, stage ^ 1);
-            if (kc + D < nchunks) {
-              JT_LOAD_W(slot, (kc + D) * kRouterKC);
-              JT_LOAD_X(slot, (kc + D) * kRouterKC);
-            }
-          }
         }
         __syncthreads();
       }
@@ -552,67 +565,66 @@ __global__ __launch_bounds__(64 * NW) void router_mfma_kernel(
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      sm.tile[(wave * 16 + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = round_to_bf16(acc[nb][i]);
+      sm.tile[(wave * 16 + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = round_to_bf16(total[nb][i]);
   __syncthreads();
   router_epilogue<bf16_raw, 16 * NW, 64 * NW>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores,
                                               logits_out, router_scratch(ws, E), score_func);
 }
 
 // ---------------------------------------------------------------------------
-// The same projection with the k range of every staged chunk shared out over the four waves
-// of a workgroup: 16 tokens per workgroup, 128 k rows per LDS stage, wave w multiplying rows
-// [32 w, 32 w + 32) of each stage.  The four partial sums are added in wave order.  A workgroup
-// then runs H/128 short iterations instead of H/64 longer ones, and 16 tokens already make a
-// workgroup, so small batches spread over more CUs.
+// Small batches: 16 tokens per workgroup, 128 k rows per LDS stage, and the four waves of a workgroup
+// share out the EXPERT COLUMNS (wave w owns the 16-column blocks w, w + 4, ...), so that each
+// accumulator still sees its k range as one chain in k order -- the summation order above.
+// A workgroup then runs H/128 short iterations instead of H/64 longer ones, and 16 tokens already
+// make a workgroup, so small batches spread over more CUs.
 // ---------------------------------------------------------------------------
-constexpr int kSplitKC = 128;
 constexpr int kSplitMaxTokens = 256;
 
-__host__ __device__ inline size_t router_split_red_offset(int E, int K) {
-  return (router_smem_bytes(E, K, 16) + 15) / 16 * 16;
-}
 __host__ __device__ inline size_t router_split_smem_bytes(int E, int K) {
   const size_t w = (size_t)2 * kSplitKC * router_w_stride(E) * 2;
-  const size_t ep = router_split_red_offset(E, K) + (size_t)4 * 16 * (E + 1) * 4;
+  const size_t ep = router_smem_bytes(E, K, 16);
   return w > ep ? w : ep;
 }
 
-// kPartial: the grid's y dimension also shares out the chunks (chunks_per_slice each); a workgroup
-// then only writes its unrounded partial sums, partial_out[slice][token][expert], and
-// router_finish_kernel adds the slices in order and does the rest.
+// kPartial: the grid's y dimension shares out the slices; a workgroup then only writes the unrounded
+// sum of its slice, partial_out[slice][token][expert], and router_finish_kernel adds the slices in
+// order and does the rest.  Otherwise the workgroup walks all slices itself.
 template <int NB, bool kPartial>
 __global__ __launch_bounds__(256) void router_mfma_split_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
     int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
     float* __restrict__ scores, float* __restrict__ logits_out, void* ws, float* __restrict__ partial_out,
-    int chunks_per_slice, int score_func) {
+    int score_func) {
   constexpr int kThreads = 256, kTokens = 16;
   constexpr int E = NB * 16;
   constexpr int WS = E + 32;
   constexpr int W_CHUNKS = kSplitKC * E / 8;
   constexpr int CW = (W_CHUNKS + kThreads - 1) / kThreads;
   constexpr int CPR = E / 8;
+  constexpr int NBW = (NB + 3) / 4;  // column blocks per wave
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint16_t* const Ws = reinterpret_cast<uint16_t*>(smem_raw);  // [2][kSplitKC][WS]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool has_cols = wave < NB;  // with fewer than four column blocks some waves only help to stage the matrix
   const int t0 = blockIdx.x * kTokens;
   const int nrows = min(kTokens, tokens - t0);
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(x + (size_t)t0 * H), 0, nrows * H * 2, kBufferFlags);
-  // lane (m = lane%16, kg = lane/16) holds k = chunk*128 + wave*32 + kg*8 + [0,8) of token t0 + m
-  const int x_voff = ((lane & 15) * H + wave * 32 + (lane >> 4) * 8) * 2;
+  // lane (m = lane%16, g = lane/16) holds k = chunk*128 + n*32 + g*8 + [0,8), n = 0..3, of token t0 + m
+  const int x_voff = ((lane & 15) * H + (lane >> 4) * 8) * 2;
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(w), 0, H * E * 2, kBufferFlags);
 
   constexpr int D = CW <= 8 ? 3 : 2;   // chunks in flight (register ring, chunk c in slot c % D)
   constexpr int UNROLL = D == 3 ? 6 : 2;
-  u32x4_t a_ring[D], w_ring[D][CW];
-  f32x4_t acc[NB];
+  u32x4_t a_ring[D][4], w_ring[D][CW];
+  f32x4_t acc[NBW], total[NBW];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
+  for (int b = 0; b < NBW; ++b)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[nb][i] = 0.0f;
+    for (int i = 0; i < 4; ++i) acc[b][i] = total[b][i] = 0.0f;
 
 #define JT_LOAD(slot, k0)                                                                     \
   {                                                                                           \
@@ -621,7 +633,10 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
       if (W_CHUNKS % kThreads == 0 || c < W_CHUNKS)                                           \
         w_ring[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c * 16, (k0)*E * 2, 0); \
     }                                                                                         \
-    a_ring[slot] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff, (k0)*2, 0);          \
+    if (has_cols) {                                                                           \
+      _Pragma("unroll") for (int n = 0; n < 4; ++n)                                           \
+        a_ring[slot][n] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff + n * 64, (k0)*2, 0); \
+    }                                                                                         \
   }
 #define JT_STORE_W(slot, stage)                                                               \
   _Pragma("unroll") for (int i = 0; i < CW; ++i) {                                            \
@@ -632,12 +647,14 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
     }                                                                                         \
   }
 
-  // transposing read: the 16-lane group kg reads rows wave*32 + kg*8 + 4*h + i/4, columns 4*(i%4)..
-  const int w_lane = (wave * 32 + (lane >> 4) * 8 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
-  // this workgroup's chunks: all of them, or one slice of them
-  const int chunk0 = kPartial ? (int)blockIdx.y * chunks_per_slice : 0;
-  const int nchunks = kPartial ? min(chunks_per_slice, H / kSplitKC - chunk0) : H / kSplitKC;
+  // transposing read: the 16-lane group g reads rows n*32 + g*8 + 4*h + i/4, columns 4*(i%4)..
+  const int w_lane = ((lane >> 4) * 8 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
+  // this workgroup's chunks: one slice of them, or all
+  const int slice_chunks = router_slice_rows(H) / kSplitKC;
+  const int chunk0 = kPartial ? (int)blockIdx.y * slice_chunks : 0;
+  const int nchunks = kPartial ? min(slice_chunks, H / kSplitKC - chunk0) : H / kSplitKC;
   const int kbase = chunk0 * kSplitKC;
+  int in_slice = 0;
 #pragma unroll
   for (int d = 0; d < D; ++d)
     if (d < nchunks) JT_LOAD(d, kbase + d * kSplitKC);
@@ -649,19 +666,37 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
       const int kc = kc0 + j;
       if (kc < nchunks) {  // uniform over the workgroup
         const int stage = j % 2, slot = j % D, next_slot = (j + 1) % D;
-        const uint16_t* wbase = Ws + stage * kSplitKC * WS + w_lane;
-        const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_ring[slot]);
+        if (has_cols) {
+          const uint16_t* wbase = Ws + stage * kSplitKC * WS + w_lane + wave * 16;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          const uint16_t* p = wbase + nb * 16;
-          const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
-          const s16x4_t hi =
-              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
-          const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[nb], 0, 0, 0);
+          for (int n = 0; n < 4; ++n) {
+            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, a_ring[slot][n]);
+#pragma unroll
+            for (int b = 0; b < NBW; ++b) {
+              const uint16_t* p = wbase + n * 32 * WS + b * 64;
+              const s16x4_t lo =
+                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+              const s16x4_t hi =
+                  __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * WS));
+              const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+              acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, both), acc[b], 0, 0, 0);
+            }
+          }
         }
         if (kc + 1 < nchunks) JT_STORE_W(next_slot, stage ^ 1);
         if (kc + D < nchunks) JT_LOAD(slot, kbase + (kc + D) * kSplitKC);
+        if (!kPartial && (++in_slice == slice_chunks || kc + 1 == nchunks)) {
+          // end of a slice: its sum joins the total, in slice order
+          const bool first = kc < slice_chunks;
+          in_slice = 0;
+#pragma unroll
+          for (int b = 0; b < NBW; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              total[b][i] = first ? acc[b][i] : total[b][i] + acc[b][i];
+              acc[b][i] = 0.0f;
+            }
+        }
         __syncthreads();
       }
     }
@@ -669,29 +704,32 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
 #undef JT_LOAD
 #undef JT_STORE_W
 
-  // partial sums of the four waves -> LDS, added in wave order, rounded to bf16 (the projection's
-  // output dtype); value i of lane l is token row 4*(l/16) + i, expert nb*16 + l%16
+  // value i of lane l of block b is token row 4*(l/16) + i, expert (wave + 4 b)*16 + l%16
+  if (kPartial) {
+    if (has_cols) {
+#pragma unroll
+      for (int b = 0; b < NBW; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = 4 * (lane >> 4) + i;
+          if (t < nrows && wave + 4 * b < NB)
+            partial_out[((size_t)blockIdx.y * tokens + t0 + t) * E + (wave + 4 * b) * 16 + (lane & 15)] = acc[b][i];
+        }
+    }
+    return;
+  }
+  // the total, rounded to bf16 (the projection's output dtype) -> LDS tile (the matrix stages are dead:
+  // the loop ends with a barrier)
   RouterSmem sm = router_smem(smem_raw, E, K, kTokens);
   const int stride = E + 1;
-  float* const red = reinterpret_cast<float*>(smem_raw + router_split_red_offset(E, K));
+  if (has_cols) {
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
+    for (int b = 0; b < NBW; ++b)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      red[(wave * kTokens + 4 * (lane >> 4) + i) * stride + nb * 16 + (lane & 15)] = acc[nb][i];
-  __syncthreads();
-  for (int idx = tid; idx < kTokens * E; idx += kThreads) {
-    const int t = idx / E, e = idx - t * E;
-    float v = red[t * stride + e];
-#pragma unroll
-    for (int wv = 1; wv < 4; ++wv) v += red[(wv * kTokens + t) * stride + e];
-    if (kPartial) {
-      if (t < nrows) partial_out[((size_t)blockIdx.y * tokens + t0 + t) * E + e] = v;
-    } else {
-      sm.tile[t * stride + e] = round_to_bf16(v);
-    }
+      for (int i = 0; i < 4; ++i)
+        if (wave + 4 * b < NB)
+          sm.tile[(4 * (lane >> 4) + i) * stride + (wave + 4 * b) * 16 + (lane & 15)] = round_to_bf16(total[b][i]);
   }
-  if (kPartial) return;
   __syncthreads();
   router_epilogue<bf16_raw, kTokens, kThreads>(sm, bias, t0, tokens, E, K, route_scale, ids, weights, scores,
                                                logits_out, router_scratch(ws, E), score_func);
@@ -705,7 +743,6 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
 // the stable permutation and its inverse) from the ids it holds in LDS; the tables of that step take
 // the place of the score tile, which is dead by then.  Requires tokens * K <= kSmallMaxAssignments
 // and E <= 4 * kTok.
-constexpr int kPartialMaxSlices = 8;
 template <int kTok, bool kPlan>
 __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
     const float* __restrict__ partial, int slices, const float* __restrict__ bias, int tokens, int E, int K,
@@ -785,9 +822,8 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
       // k slices from many workgroups, then the finishing workgroup.
       const int finish_tok = router_smem_bytes((int)E, (int)K, 256) <= 160 * 1024 ? 256 : 64;
       if (tokens > 0 && tokens <= finish_tok && router_smem_bytes((int)E, (int)K, finish_tok) <= 160 * 1024) {
-        const int chunks = (int)(H / kSplitKC);
-        const int per_slice = (chunks + kPartialMaxSlices - 1) / kPartialMaxSlices;
-        const int slices = (chunks + per_slice - 1) / per_slice;
+        const int slice_rows = router_slice_rows((int)H);
+        const int slices = (int)((H + slice_rows - 1) / slice_rows);
         float* partial = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + router_scratch_bytes(E));
 #define JT_PARTIAL_CASE(NB)                                                                                   \
   case NB * 16: {                                                                                            \
@@ -796,7 +832,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (rc) return rc;                                                                                       \
     kernel<<<dim3(blocks, slices), 256, smem, stream>>>(                                                     \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws, partial, per_slice, \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws, partial,           \
         score_func);                                                                                         \
   } break;
         switch ((int)E) {
@@ -841,7 +877,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
     if (rc) return rc;                                                                                       \
     kernel<<<blocks, 256, smem, stream>>>(                                                                   \
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), bias, (int)tokens, (int)H, (int)K, \
-        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats, nullptr, 0,  \
+        (float)route_scale, ids, static_cast<bf16_raw*>(weights), scores, logits_out, ws_stats, nullptr,     \
         score_func);                                                                                         \
   } break;
         switch ((int)E) {

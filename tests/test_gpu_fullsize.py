@@ -79,12 +79,16 @@ def test_full_size_rows_match_sub_batch_and_oracle_sample(c3, gpu):
     rng = np.random.default_rng(0)
     pick = np.sort(rng.choice(T, size=96, replace=False))
     sub = run(c3, x=c3["x"][torch.from_numpy(pick).to(gpu)].contiguous())
-    # a batch this small takes the router kernel that splits the k range over the waves: its logits can
-    # differ from the large-batch kernel's in the last bit, which may flip a near-tie
-    same = (host(sub.expert_ids) == host(full.expert_ids)[pick]).all(axis=1)
-    assert same.mean() >= 0.97
-    assert np.array_equal(host(sub.weights)[same], host(full.weights)[pick][same])
-    assert rel_err(host(sub.y)[same], host(full.y)[pick][same]) <= 1e-2
+    # A batch this small takes other router kernels (the k range shared out over workgroups) than the full
+    # batch; all of them add a logit up in one order, so a token routes the same whatever shares its call
+    # (the reference's invariant prefill + decode == full forward, tests/jaxtitan/test_infer.py:270-301).
+    for name in ("expert_ids", "weights", "scores"):
+        a, b = host(getattr(sub, name)), host(getattr(full, name))[pick]
+        assert np.array_equal(a, b), f"{name}: {int((a != b).any(axis=1).sum())} of {len(pick)} rows differ from the full batch"
+    err = rel_err(host(sub.y), host(full.y)[pick])
+    print(f"[parity] {c3['name']} 96-token sub-batch against the same rows of the full batch: routing identical, "
+          f"y max_rel={err:.3e}", flush=True)
+    assert err <= 1e-2
     # the oracle on the same tokens, with the kernel's routing
     inp = c3["inp"]
     x2 = inp["x"].reshape(T, cfg["H"])[pick]

@@ -414,9 +414,30 @@ def check_layer_against_oracle(gpu, inp, top_k, dtype, tag):
     E = inp["gate"].shape[0]
     ids = host(got.expert_ids)
     ref_route = O.router(x2, inp["w_router"], inp["expert_bias"], top_k, 1.0, dtype)
-    mism = int(np.sum(np.any(ids != ref_route.expert_ids, axis=1)))
-    print(f"[parity] {tag}: tokens routed differently from the oracle's own logits: {mism}/{x2.shape[0]}", flush=True)
-    assert mism <= max(1, x2.shape[0] // 500)
+    # Routing against the oracle: a row may route differently only where one of its logits differs from the
+    # oracle's (two fp32 summation orders, then one rounding to the compute dtype, so by one unit in the last
+    # place at most), and the layer's decision is the oracle's decision on the kernel's own logits -- which
+    # the stand-alone router call returns and the layer call does not.
+    alone = ops.router(dev(x2, gpu, dtype), dev(inp["w_router"], gpu, dtype), dev(inp["expert_bias"], gpu), top_k, 1.0,
+                       return_logits=True)
+    assert np.array_equal(host(alone.expert_ids), ids) and np.array_equal(host(alone.scores), host(got.scores))
+    logits = host(alone.logits)
+    ulp = np.maximum(np.abs(ref_route.logits) * 2.0**-7, 1e-5) if dtype == "bf16" else np.abs(ref_route.logits) * 2e-5 + 2e-6
+    assert np.all(np.abs(logits - ref_route.logits) <= ulp)
+    own = O.router_from_logits(logits, inp["expert_bias"], top_k, 1.0, dtype)
+    assert np.array_equal(ids, own.expert_ids) and np.array_equal(host(got.weights), own.weights)
+    other_logit = np.any(logits != ref_route.logits, axis=1)
+    flipped = np.any(ids != ref_route.expert_ids, axis=1)
+    print(f"[parity] {tag}: of {x2.shape[0]} tokens {int(other_logit.sum())} have a logit that differs from the "
+          f"oracle's in the last place ({int((logits != ref_route.logits).sum())} of {logits.size} logits), "
+          f"{int(flipped.sum())} of them route differently", flush=True)
+    assert not np.any(flipped & ~other_logit), "a token with the oracle's logits routes differently"
+    # bf16: two fp32 sums of H terms differ by some 2^-20 of their size and a bf16 rounding boundary lies
+    # every 2^-8, so about 2^-12 of the logits fall on the other side of one (measured: 1.2e-4 at the second
+    # configuration's shape, 2.2e-4 at the third's).  fp32 logits differ in their last bits wherever the two
+    # summation orders do, and no score is within reach of another.
+    if dtype == "bf16":
+        assert int((logits != ref_route.logits).sum()) <= max(2, logits.size // 1000)
     d = O.dispatch(ids, E, O.cast_compute(x2, dtype))
     assert np.array_equal(host(got.group_sizes), d.group_sizes)
     assert np.array_equal(host(got.offsets), d.offsets)

@@ -15,7 +15,7 @@ import test_gpu_parity as P  # the tests directory is on sys.path under pytest (
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("seed", [11, 12])
+@pytest.mark.parametrize("seed", [11, 12, 13, 14])
 def test_random_router_shapes(gpu, seed):
     rng = np.random.default_rng(seed)
     for _ in range(24):
@@ -32,7 +32,7 @@ def test_random_router_shapes(gpu, seed):
         P.check_router_end_to_end(gpu, x, w, bias, top_k, float(rng.choice([1.0, 2.5])), dtype)
 
 
-@pytest.mark.parametrize("seed", [21, 22])
+@pytest.mark.parametrize("seed", [21, 22, 23, 24])
 def test_random_dispatch_shapes(gpu, seed):
     rng = np.random.default_rng(seed)
     for _ in range(24):
@@ -49,7 +49,7 @@ def test_random_dispatch_shapes(gpu, seed):
         P.check_dispatch(gpu, ids, experts, x, dtype)
 
 
-@pytest.mark.parametrize("seed", [31])
+@pytest.mark.parametrize("seed", [31, 32, 33, 34])
 def test_random_expert_and_combine_shapes(gpu, seed):
     rng = np.random.default_rng(seed)
     for _ in range(16):
@@ -70,7 +70,7 @@ def test_random_expert_and_combine_shapes(gpu, seed):
         P.test_combine_is_bit_exact(gpu, tokens, hidden, top_k, dtype, bool(rng.random() < 0.5))
 
 
-@pytest.mark.parametrize("seed", [41])
+@pytest.mark.parametrize("seed", [41, 42, 43, 44, 1001, 1012])
 def test_random_gradient_shapes(gpu, seed):
     """The backward operators on odd shapes: rows that leave the fast GEMM paths, single tokens,
     one expert, top_k = num_experts."""
