@@ -260,7 +260,11 @@ int jtmoe_smebu_update(const float* router_counts, float* momentum, float* exper
  *   out: y [T,H]; expert_ids [T,K]; weights [T,K]; scores [T,E];
  *        expert_counts, importance [E] f32; group_sizes, offsets [E] i32;
  *        source_order, inverse [A] i32.
- *   workspace: jtmoe_workspace_bytes(...) bytes, 256-byte aligned.
+ *   workspace: jtmoe_workspace_bytes(...) bytes, 256-byte aligned.  Where
+ *        jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) holds, the grouped
+ *        GEMM fetches its rows through the permutation, the workspace holds no
+ *        permuted copy of x ([A,H]: a third of it at 64 experts, top-8, H = 2048),
+ *        and x, gate, up and down must be 16-byte aligned (JTMOE_EINVAL otherwise).
  */
 size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype);
 int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_bias,

@@ -4,6 +4,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 namespace jtmoe {
 
@@ -305,6 +306,35 @@ __global__ __launch_bounds__(kSmebuWaves * 64) void smebu_update_kernel(
   }
 }
 
+// A second stream per device, with the two events of a fork and join, for the one place where the
+// layer has independent work to overlap (the decode path: expert matrices streamed beside the router).
+// Default priority, created on the first use on a device and kept until the process ends.  The
+// events carry no timing; a wait takes the state of its event at the moment it is enqueued, so the
+// pair can be recorded again by the next call (the mutex covers one call's fork ... join sequence).
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  bool ok = false, tried = false;
+};
+constexpr int kMaxDevices = 64;
+std::mutex g_side_mutex;
+SideStream g_side[kMaxDevices];
+
+// with g_side_mutex held
+SideStream* side_stream_locked() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+  SideStream& sd = g_side[device];
+  if (!sd.tried) {
+    sd.tried = true;
+    sd.ok = hipStreamCreateWithFlags(&sd.stream, hipStreamNonBlocking) == hipSuccess &&
+            hipEventCreateWithFlags(&sd.fork, hipEventDisableTiming) == hipSuccess &&
+            hipEventCreateWithFlags(&sd.join, hipEventDisableTiming) == hipSuccess;
+    if (!sd.ok) (void)hipGetLastError();  // the caller falls back to one stream
+  }
+  return sd.ok ? &sd : nullptr;
+}
+
 struct Carve {
   unsigned char* base;
   size_t used;
@@ -337,8 +367,12 @@ LayerWorkspace carve_layer(void* base, int64_t T, int64_t H, int64_t E, int64_t 
   w.router = c.take(w.router_bytes);
   w.dispatch_bytes = dispatch_layer_workspace_bytes((int64_t)A, E);
   w.dispatch = c.take(w.dispatch_bytes);
-  w.packed_x = c.take(A * (size_t)H * b);
-  w.act = c.take(A * (size_t)I * b);
+  // the permuted copy of x exists only where the grouped GEMM cannot fetch its rows through the
+  // permutation itself (a third of the workspace at 64 experts x top-8 x 2048)
+  w.packed_x = jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) ? nullptr : c.take(A * (size_t)H * b);
+  // (the decode path keeps the activations of all tokens through every expert)
+  const size_t act_rows = decode_dense_supported(T, H, E, K, I, dtype) ? (size_t)E * (size_t)T : A;
+  w.act = c.take((act_rows > A ? act_rows : A) * (size_t)I * b);
   w.packed_y = c.take(A * (size_t)H * b);
   w.shared_act = Is > 0 ? c.take((size_t)T * (size_t)Is * b) : nullptr;
   w.shared_y = Is > 0 ? c.take((size_t)T * (size_t)H * b) : nullptr;
@@ -451,25 +485,71 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
   const LayerWorkspace w = carve_layer(workspace, T, H, E, K, I, Is, dtype);
   if (workspace_bytes < w.total)
     return fail(JTMOE_EWORKSPACE, "moe_forward: workspace %zu < %zu bytes", workspace_bytes, w.total);
+  // where the GEMM can apply the permutation while it fetches its A tiles, the permuted copy of
+  // x is never written: dispatch then only computes the histogram, offsets and permutation
+  const bool gather = train || (T > 0 && jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype));
+  // the workspace of such a shape holds no permuted copy of x to fall back on
+  if (gather && !train &&
+      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up) |
+        reinterpret_cast<uintptr_t>(down)) & 15u) != 0)
+    return fail(JTMOE_EINVAL, "moe_forward: x and the expert matrices must be 16-byte aligned");
   // The router of a layer call leaves out what the dispatch behind it can do in passing: at large
   // batches the statistics (no zeroing and no finalising launch, no global atomics), at small ones
   // its finishing workgroup writes the dispatch plan as well.
+  // Decode path (a handful of tokens): the gate/up launch runs every token through every expert, which
+  // needs nothing of the routing, so the router (and the plan) run beside it on a second stream; the
+  // down launch then picks the routed rows.  The GEMM stays on the caller's stream and the router goes
+  // to the other one, not the reverse: a dependency that crosses streams costs about 10 us when the
+  // waiting stream is idle at that moment, and the router's result is there long before the GEMM ends.
+  // With a stage timer installed everything stays on the one stream, so that a stage's time is its
+  // kernels' time.
+  hipStream_t main_stream = as_stream(stream);
+  const bool decode = !train && decode_dense_supported(T, H, E, K, I, dtype);
+  std::unique_lock<std::mutex> side_lock(g_side_mutex, std::defer_lock);  // held from the fork to the join
+  SideStream* side = nullptr;
+  if (decode && g_stage_timer == nullptr) {
+    side_lock.lock();
+    side = side_stream_locked();
+    if (side != nullptr && (hipEventRecord(side->fork, main_stream) != hipSuccess ||
+                            hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)) {
+      (void)hipGetLastError();
+      side = nullptr;
+    }
+    if (side == nullptr) side_lock.unlock();
+  }
+  const bool forked = side != nullptr;
+  hipStream_t route_stream = forked ? side->stream : main_stream;
   bool stats_done = false, plan_done = false;
-  int rc = router_for_layer(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
-                            expert_counts, importance, group_sizes, offsets, source_order, inverse, w.router,
-                            w.router_bytes, score_func, &stats_done, &plan_done, as_stream(stream));
+  // (forked: the expert matrices start streaming on the caller's stream before anything else is enqueued)
+  int rc = forked ? launch_gate_up_all_tokens(x, gate, up, w.act, T, H, I, E, main_stream) : JTMOE_OK;
+  if (rc == JTMOE_OK)
+    rc = router_for_layer(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
+                          expert_counts, importance, group_sizes, offsets, source_order, inverse, w.router,
+                          w.router_bytes, score_func, &stats_done, &plan_done, route_stream, forked);
+  if (rc == JTMOE_OK) {
+    stage_mark(kStageRouter, route_stream);
+    rc = dispatch_for_layer(expert_ids, weights, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes,
+                            offsets, source_order, inverse, w.packed_x, expert_counts, importance, w.dispatch,
+                            !stats_done, plan_done, route_stream);
+  }
+  if (forked) {
+    // the second stream joins again whatever happened on it (a capture of the caller's stream could not end otherwise)
+    const bool joined = hipEventRecord(side->join, side->stream) == hipSuccess &&
+                        hipStreamWaitEvent(main_stream, side->join, 0) == hipSuccess;
+    side_lock.unlock();
+    if (rc == JTMOE_OK && !joined) rc = fail(JTMOE_ELAUNCH, "moe_forward: joining the second stream failed");
+  }
   if (rc) return rc;
-  stage_mark(kStageRouter, as_stream(stream));
-  // where the GEMM can apply the permutation while it fetches its A tiles, the permuted copy of
-  // x is never written: dispatch then only computes the histogram, offsets and permutation
-  const bool gather = train || (T > 0 && jtmoe_grouped_swiglu_gather_supported(T, H, I, dtype) &&
-                      (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(gate) & 15u) == 0 &&
-                      (reinterpret_cast<uintptr_t>(up) & 15u) == 0 && (reinterpret_cast<uintptr_t>(down) & 15u) == 0);
-  rc = dispatch_for_layer(expert_ids, weights, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes,
-                          offsets, source_order, inverse, w.packed_x, expert_counts, importance, w.dispatch,
-                          !stats_done, plan_done, as_stream(stream));
-  if (rc) return rc;
-  if (train)
+  if (decode) {
+    if (!forked) rc = launch_gate_up_all_tokens(x, gate, up, w.act, T, H, I, E, main_stream);
+    if (rc) return rc;
+    stage_mark(kStageGateUp, main_stream);
+    rc = launch_down_from_all_tokens(w.act, down, group_sizes, offsets, source_order, T, K, H, I, E, w.packed_y,
+                                     main_stream);
+    if (rc) return rc;
+    stage_mark(kStageDown, main_stream);
+    rc = check_launch("grouped gemm");
+  } else if (train)
     rc = jtmoe_grouped_swiglu_train(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
                                     gate_pre, up_pre, w.act, w.packed_y, stream);
   else if (gather)

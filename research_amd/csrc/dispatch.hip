@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(const int32
       const int id = ids[a];
       if (id >= 0 && id < E) {
         atomicAdd(&hist[id], 1);
-        if (kStats) atomicAdd(&imp[id], (unsigned long long)(Elem<WT>::load(weights + a) * kImportanceScale));
+        if (kStats) atomicAdd(&imp[id], importance_term(Elem<WT>::load(weights + a)));
       }
     }
   }

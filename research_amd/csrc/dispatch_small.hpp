@@ -15,6 +15,14 @@ namespace jtmoe {
 constexpr int kSmallMaxAssignments = 8192;
 constexpr int kSmallMaxExperts = JTMOE_MAX_EXPERTS;
 constexpr float kImportanceScale = 4294967296.0f;  // importance is summed in 32.32 fixed point: any order, same sum
+// A route weight as a 32.32 fixed-point term.  Route weights are finite, non-negative and far below 2^32
+// (at most route_scale); anything else (a NaN from non-finite logits, a negative or huge value handed
+// to the dispatcher by a caller) would make the float -> integer conversion undefined, so NaN and
+// negative values count as 0 and the rest is clamped to the largest float below 2^32.
+__device__ __forceinline__ unsigned long long importance_term(float w) {
+  w = fminf(fmaxf(w, 0.0f), 4294967040.0f);  // fmaxf(NaN, 0) = 0
+  return (unsigned long long)(w * kImportanceScale);
+}
 
 // LDS of the body: cursor[E], wavehist[waves][E], wave_sums[waves] ints, then (kStats) imp[E] of 8 bytes
 __host__ __device__ inline size_t dispatch_small_smem_bytes(int E, int threads, bool stats) {
@@ -52,7 +60,7 @@ __device__ __forceinline__ void dispatch_small_body(const int32_t* ids, const WT
     const int id = ids[a];
     if (id >= 0 && id < E) {
       atomicAdd(&cursor[id], 1);
-      if (kStats) atomicAdd(&imp[id], (unsigned long long)(Elem<WT>::load(weights + a) * kImportanceScale));
+      if (kStats) atomicAdd(&imp[id], importance_term(Elem<WT>::load(weights + a)));
     }
   }
   __syncthreads();

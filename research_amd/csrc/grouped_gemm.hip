@@ -159,7 +159,7 @@ template <typename Cfg>
 int launch_fast(const void* a, const void* b0, const void* b1, void* c, const int32_t* group_sizes,
                 const int32_t* offsets, int64_t rows, int64_t Kdim, int64_t N, int64_t E, hipStream_t stream,
                 const int32_t* row_map = nullptr, int row_div = 1, int64_t a_rows = 0, void* save0 = nullptr,
-                void* save1 = nullptr) {
+                void* save1 = nullptr, int64_t uniform_rows = 0, int64_t a_group_rows = 0) {
   // the 256-row configurations run as persistent workgroups (see persistent_schedule), the others one
   // tile per workgroup
   constexpr bool kPersistent = Cfg::BM == 256 && Cfg::NSTAGE == 2 && Cfg::BK == 64;
@@ -178,11 +178,15 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
   if (attr_err != hipSuccess)
     return fail(JTMOE_ELAUNCH, "grouped gemm: kernel set-up: %s", hipGetErrorString(attr_err));
   const bool dense = group_sizes == nullptr;
-  const int64_t mtiles = dense ? (rows + Cfg::BM - 1) / Cfg::BM : max_m_tiles(rows, E, Cfg::BM);
+  const int64_t mtiles = uniform_rows > 0 ? E * ((uniform_rows + Cfg::BM - 1) / Cfg::BM)
+                         : dense          ? (rows + Cfg::BM - 1) / Cfg::BM
+                                          : max_m_tiles(rows, E, Cfg::BM);
   const int64_t nt = (N + Cfg::BN - 1) / Cfg::BN;
   const int64_t tiles_grid = gemm_grid(mtiles, nt);
   if (tiles_grid >= ((int64_t)1 << 31)) return fail(JTMOE_EUNSUPPORTED, "grouped gemm: grid too large");
   if constexpr (kPersistent) {
+    if (uniform_rows > 0 || a_group_rows > 0)
+      return fail(JTMOE_EUNSUPPORTED, "grouped gemm: the decode forms run one tile per workgroup");
     const PersistentSchedule ps = persistent_schedule(tiles_grid, persistent_grid_size(), kTilesPerWorkgroup<Cfg>);
     kernel<<<(unsigned)ps.grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
         static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
@@ -193,7 +197,8 @@ int launch_fast(const void* a, const void* b0, const void* b1, void* c, const in
     kernel<<<(unsigned)tiles_grid, Cfg::NT, Cfg::SMEM_BYTES, stream>>>(
         static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b0), static_cast<const uint16_t*>(b1),
         static_cast<uint16_t*>(c), group_sizes, offsets, (int)E, (int)rows, (int)Kdim, (int)N, (int)mtiles, (int)nt,
-        row_map, row_div, (int)a_rows, static_cast<uint16_t*>(save0), static_cast<uint16_t*>(save1));
+        row_map, row_div, (int)a_rows, static_cast<uint16_t*>(save0), static_cast<uint16_t*>(save1), (int)uniform_rows,
+        (int)a_group_rows);
   }
   return JTMOE_OK;
 }
@@ -298,6 +303,34 @@ int validate_gemm(const char* what, int64_t rows, int64_t H, int64_t I, int64_t 
 }
 
 }  // namespace
+
+// ---- the decode path of the layer (declared in common.hpp) ----
+constexpr int64_t kDecodeMaxTokens = 64;  // one 64-row tile per expert holds every token
+
+bool decode_dense_supported(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype) {
+  // all tokens through every expert pays when nearly every expert would be streamed anyway: with
+  // T * K >= 2 E assignments thrown at E experts fewer than e^-2 = 14 % of them stay without a row
+  return dtype == JTMOE_BF16 && T > 0 && T <= kDecodeMaxTokens && T * K >= 2 * E && tiny_groups(T * K, E) &&
+         E <= JTMOE_MAX_EXPERTS && H % 64 == 0 && I % 64 == 0 && H * I < ((int64_t)1 << 30) &&
+         E * T * (I > H ? I : H) < ((int64_t)1 << 30);
+}
+
+int launch_gate_up_all_tokens(const void* x, const void* gate, const void* up, void* act_full, int64_t T, int64_t H,
+                              int64_t I, int64_t E, hipStream_t stream) {
+  if (!fast_ok(x, gate, up, act_full, H, I)) return fail(JTMOE_EINVAL, "moe_forward: operands must be 16-byte aligned");
+  return launch_fast<GateUpTinyCfg>(x, gate, up, act_full, nullptr, nullptr, E * T, H, I, E, stream, nullptr, 1, 0,
+                                    nullptr, nullptr, /*uniform_rows=*/T);
+}
+
+int launch_down_from_all_tokens(const void* act_full, const void* down, const int32_t* group_sizes,
+                                const int32_t* offsets, const int32_t* source_order, int64_t T, int64_t K, int64_t H,
+                                int64_t I, int64_t E, void* packed_y, hipStream_t stream) {
+  if (!fast_ok(act_full, down, nullptr, packed_y, I, H))
+    return fail(JTMOE_EINVAL, "moe_forward: operands must be 16-byte aligned");
+  return launch_fast<DownTinyCfg>(act_full, down, nullptr, packed_y, group_sizes, offsets, T * K, I, H, E, stream,
+                                  source_order, (int)K, T, nullptr, nullptr, 0, /*a_group_rows=*/T);
+}
+
 }  // namespace jtmoe
 
 using namespace jtmoe;

@@ -30,6 +30,8 @@
 
 #include "gemm_common.hpp"
 
+#include <type_traits>
+
 namespace jtmoe {
 
 typedef __attribute__((ext_vector_type(4))) int i32x4_t;
@@ -103,7 +105,8 @@ struct DmaGemmCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NSTAGE = NSTAGE_;
   // scheduling options: 16 = request the fragments of MFMA step kk+1 before issuing step kk,
   // 32 = raise the wave priority around the MFMA burst, 64 = ask the scheduler to interleave
-  // one MFMA with up to three LDS reads, 128 = B tiles in 4 x 64 blocks, 4096 = non-temporal loads of B, 32768 = non-temporal stores of the result
+  // one MFMA with up to three LDS reads, 128 = B tiles in 4 x 64 blocks, 2048 = (persistent kernel) results written
+  // straight from transposed accumulators instead of through LDS, 4096 = non-temporal loads of B, 32768 = non-temporal stores of the result
   static constexpr int OPT = OPT_;
   static constexpr bool kDual = kDual_;
   static constexpr int BNE = kDual ? 2 * BN : BN;  // columns of the B tile in LDS
@@ -135,12 +138,102 @@ struct DmaGemmCfg {
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
+// two fp32 values -> their bf16 roundings packed in one dword (lo in the low half): one hardware conversion
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+
+// Epilogue of the kernels that issue their MFMAs with the WEIGHT fragment as the first operand: a
+// 32 x 32 accumulator then holds the TRANSPOSED block -- value i of lane l is row l % 32, column
+// 8 * (i / 4) + 4 * (l / 32) + i % 4 of the block, i.e. a lane owns runs of four neighbouring columns
+// of one row.  Two such runs are packed to bf16 pairs, the half-waves swap one of them
+// (v_permlane32_swap), and every lane stores 16 contiguous bytes: no LDS staging, no barrier.
+// Stores go through a buffer descriptor of the whole result (out_rows_total rows of N columns, at most
+// 0x7ffe0000 bytes): one 32-bit offset per row, the column of each store as an immediate, and rows
+// past the end of the group (or columns past N) get the offset 0x7fff0000, which lies outside every
+// admitted result, so the hardware drops the store.
+// With save0 / save1 (dual tiles only) the two rounded products are written as well.
+template <typename Cfg>
+__device__ __forceinline__ void store_transposed_accumulators(const f32x16_t (&acc)[Cfg::TM][Cfg::TN], int wm, int wn,
+                                                              int row0, int rows, int n0, int N, int out_rows_total,
+                                                              uint16_t* __restrict__ C, uint16_t* __restrict__ save0,
+                                                              uint16_t* __restrict__ save1) {
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, TNO = Cfg::TNO, WNO = Cfg::WNO;
+  constexpr bool kDual = Cfg::kDual;
+  // (the lane id is taken afresh so that nothing of the epilogue's addressing is kept in registers
+  // through the k loops, where every register is spoken for)
+  int lane_e;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
+  const int col0 = n0 + wn * WNO;
+  const int half = lane_e >> 5;
+  const int cols_left = N - (col0 + 8 * half);
+  auto write_pass = [&](auto pass_tag) {
+    constexpr int pass = decltype(pass_tag)::value;  // 0: the result, 1 and 2: the two rounded products
+    uint16_t* const out = pass == 0 ? C : (pass == 1 ? save0 : save1);
+    const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(out, 0, out_rows_total * N * 2, kBufferFlags);
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi) {
+      const int r = wm * WM + mi * 32 + (lane_e & 31);
+      const int row_off = r < rows ? ((row0 + r) * N + col0 + 8 * half) * 2 : 0x7fff0000;
+#pragma unroll
+      for (int jj = 0; jj < TNO; ++jj) {
+#pragma unroll
+        for (int qq = 0; qq < 4; qq += 2) {
+          unsigned pk[2][2];
+#pragma unroll
+          for (int dq = 0; dq < 2; ++dq) {
+#pragma unroll
+            for (int tp = 0; tp < 2; ++tp) {  // two neighbouring columns at a time
+              const int i = (qq + dq) * 4 + tp * 2;
+              if (kDual) {
+                // both products rounded to bf16 (one packed conversion each), then silu(g) * u on them
+                const unsigned gb = pack_bf16x2(acc[mi][jj][i], acc[mi][jj][i + 1]);
+                const unsigned ub = pack_bf16x2(acc[mi][jj + TN / 2][i], acc[mi][jj + TN / 2][i + 1]);
+                if (pass == 0) {
+                  const float g0 = __uint_as_float(gb << 16), g1 = __uint_as_float(gb & 0xffff0000u);
+                  const float u0 = __uint_as_float(ub << 16), u1 = __uint_as_float(ub & 0xffff0000u);
+                  pk[dq][tp] = pack_bf16x2(silu_rcp(g0) * u0, silu_rcp(g1) * u1);
+                } else {
+                  pk[dq][tp] = pass == 1 ? gb : ub;
+                }
+              } else {
+                pk[dq][tp] = pack_bf16x2(acc[mi][jj][i], acc[mi][jj][i + 1]);
+              }
+            }
+          }
+          // before: this lane has columns 8 qq + 4 half + 0..3 (pk[0]) and 8 (qq + 1) + 4 half + 0..3
+          // (pk[1]); after: columns 8 (qq + half) + 0..7
+          const auto lo = __builtin_amdgcn_permlane32_swap(pk[0][0], pk[1][0], false, false);
+          const auto hi = __builtin_amdgcn_permlane32_swap(pk[0][1], pk[1][1], false, false);
+          const u32x4_t val = {lo[0], hi[0], lo[1], hi[1]};
+          const int col = jj * 32 + 8 * qq;  // + 8 * half, already in row_off
+          const int off = col < cols_left ? row_off : 0x7fff0000;
+          // plain stores: a 128-byte line of the result is put together from four of these stores in the
+          // L2 (as non-temporal stores the 32-byte pieces cost 17 % of the down projection)
+          __builtin_amdgcn_raw_buffer_store_b128(val, out_rsrc, off + col * 2, 0, 0);
+          // keeps the compiler from computing many column runs at once (register pressure)
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  };
+  write_pass(std::integral_constant<int, 0>{});
+  if (kDual && save0 != nullptr) {
+    write_pass(std::integral_constant<int, 1>{});
+    write_pass(std::integral_constant<int, 2>{});
+  }
+}
+
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
     uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
     int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
-    int a_rows, uint16_t* __restrict__ save0 = nullptr, uint16_t* __restrict__ save1 = nullptr) {
+    int a_rows, uint16_t* __restrict__ save0 = nullptr, uint16_t* __restrict__ save1 = nullptr, int uniform_rows = 0,
+    int a_group_rows = 0) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, NSTAGE = Cfg::NSTAGE;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   constexpr int CPRA = Cfg::CPRA;
@@ -150,7 +243,19 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   // the grid covers an upper bound of the m-tiles; the tile order is cut from their real number
   TileCoord tc;
   TileRows tr;
-  if (group_sizes) {
+  int a_row0;  // first row of the tile inside A (without a row map)
+  if (uniform_rows > 0) {
+    // Every group takes the SAME uniform_rows rows of A (all tokens through every expert: the decode
+    // path, which does not wait for the routing): group e writes rows [e, e + 1) * uniform_rows of C.
+    const int per_group = (uniform_rows + BM - 1) / BM;
+    tc = xcd_tile_order(E * per_group, ntiles_n, Cfg::GROUP_M);
+    if (tc.mt < 0) return;
+    tr.expert = tc.mt / per_group;
+    const int local_row0 = (tc.mt - tr.expert * per_group) * BM;
+    tr.row0 = tr.expert * uniform_rows + local_row0;
+    tr.rows = min(BM, uniform_rows - local_row0);
+    a_row0 = local_row0;
+  } else if (group_sizes) {
     const GroupScan scan = group_scan(BM, group_sizes, E);
     tc = xcd_tile_order_balanced(scan.total, ntiles_n, Cfg::GROUP_M);
     if (tc.mt < 0) return;
@@ -160,6 +265,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
     if (tc.mt < 0) return;
     tr = find_tile_wave(tc.mt, BM, nullptr, nullptr, E, dense_rows);
   }
+  if (uniform_rows <= 0) a_row0 = tr.row0;
+  a_row0 = __builtin_amdgcn_readfirstlane(a_row0);
   const int nt = tc.nt;
   tr.expert = __builtin_amdgcn_readfirstlane(tr.expert);
   tr.row0 = __builtin_amdgcn_readfirstlane(tr.row0);
@@ -180,9 +287,11 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
   // Without a row map, tile row r is row tr.row0 + r of A.  With one (gather on load), it is row
   // row_map[tr.row0 + r] / row_div of A: the expert-major permutation is applied while the tile is
   // fetched, so the permuted copy of the activations never exists in memory.
+  // (a_group_rows > 0: A holds a block of a_group_rows rows per group, and the map's rows are rows of the
+  // tile's group's block -- the activations of the decode path above, [E][tokens][K])
   const bool gather = row_map != nullptr;
-  const i32x4_t a_rsrc = gather ? make_rsrc(A, a_rows * Kdim * 2)
-                                : make_rsrc(A + (size_t)tr.row0 * Kdim, tr.rows * Kdim * 2);
+  const i32x4_t a_rsrc = gather ? make_rsrc(A + (size_t)tr.expert * a_group_rows * Kdim, a_rows * Kdim * 2)
+                                : make_rsrc(A + (size_t)a_row0 * Kdim, tr.rows * Kdim * 2);
   // A: slot s = j*NT + tid -> row s / CPRA, slot-in-row s % CPRA holds source chunk c
   const int a_r = tid / CPRA, a_slot = tid - a_r * CPRA;
   const int a_c = a_slot ^ ((a_r / (16 / CPRA)) % CPRA);
@@ -410,6 +519,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
   constexpr int CPRA = Cfg::CPRA;
   constexpr bool kDual = Cfg::kDual;
   static_assert(Cfg::NSTAGE == 2, "two stages");
+  // results straight from (transposed) accumulators: the weight fragment is the MFMA's first operand
+  constexpr bool kDirect = (Cfg::OPT & 2048) != 0;
   extern __shared__ __align__(16) unsigned char smem_raw[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -600,7 +711,8 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
         for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
           for (int jj = 0; jj < TN; ++jj)
-            acc[mi][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
+            acc[mi][jj] = kDirect ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[kk & 1][jj], af[kk & 1][mi], acc[mi][jj], 0, 0, 0)
+                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][mi], bf[kk & 1][jj], acc[mi][jj], 0, 0, 0);
         if (Cfg::OPT & 64) {
 #pragma unroll
           for (int g = 0; g < TM * TN; ++g) {
@@ -619,6 +731,12 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_persistent_kernel(
       issue(0);
     }
 
+    if constexpr (kDirect) {
+      store_transposed_accumulators<Cfg>(acc, wm, wn, out_row0, out_rows, out_n0, N, dense_rows, C, save0, save1);
+      if (nxt.rows <= 0) break;
+      cur = nxt;
+      continue;
+    }
     const int col0 = out_n0 + wn * WNO;
     const int passes = (kDual && save0 != nullptr) ? 3 : 1;
     for (int pass = 0; pass < passes; ++pass) {

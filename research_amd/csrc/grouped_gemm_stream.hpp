@@ -35,14 +35,6 @@ __device__ __forceinline__ void buffer_load_lds4(i32x4_t rsrc, unsigned lds_base
                : "memory", "m0");
 }
 
-// two fp32 values -> their bf16 roundings packed in one dword (lo in the low half): one hardware conversion
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
-  const f32x2_t v = {lo, hi};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
-}
-
 template <typename Cfg>
 struct StreamLayout {
   static constexpr int kRowBufBytes = Cfg::NT * 4;
@@ -273,8 +265,6 @@ __device__ __forceinline__ void stream_gemm_body(
     for (int jj = 0; jj < TN; ++jj) bf[jj] = load_frag_b(stage, kk, jj);
   };
 
-  constexpr int TNO = Cfg::TNO, WNO = Cfg::WNO;
-
   // ---- first tile: plan, all NS stages requested, first fragments read ----
   Tile cur = locate(idx);
   if (cur.rows <= 0) return;
@@ -416,78 +406,8 @@ __device__ __forceinline__ void stream_gemm_body(
       __builtin_amdgcn_sched_barrier(0);
     }
 
-    // ---- epilogue: straight from the accumulators to memory ----
-    // The MFMAs take the weight fragment as their first operand, so a 32 x 32 accumulator holds the
-    // TRANSPOSED block: value i of lane l is row l % 32, column 8 * (i / 4) + 4 * (l / 32) + i % 4 of
-    // the block, i.e. a lane owns runs of four neighbouring columns of one row.  Two such runs are
-    // packed to bf16 pairs, the half-waves swap one of them (v_permlane32_swap), and every lane
-    // stores 16 contiguous bytes; no LDS staging, no barrier.
-    // Stores go through a buffer descriptor of the whole result: one 32-bit offset per row, the
-    // column of each store as an immediate, and rows past the end of the group (or columns past N)
-    // get the offset 0x7fff0000, which lies outside every result the host admits (at most 0x7ffe0000
-    // bytes), so the hardware drops the store.
-    // (the lane id is taken afresh so that nothing of the epilogue's addressing is kept in registers
-    // through the k loops, where every register is spoken for)
-    int lane_e;
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
-    const int col0 = cur.n0 + wn * WNO;
-    const int half = lane_e >> 5;
-    const int cols_left = N - (col0 + 8 * half);
-    auto write_pass = [&](auto pass_tag) {
-      constexpr int pass = decltype(pass_tag)::value;  // 0: the result, 1 and 2: the two rounded products
-      uint16_t* const out = pass == 0 ? C : (pass == 1 ? save0 : save1);
-      const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(out, 0, dense_rows * N * 2, kBufferFlags);
-#pragma unroll
-      for (int mi = 0; mi < TM; ++mi) {
-        const int r = wm * WM + mi * 32 + (lane_e & 31);
-        const int row_off = r < cur.rows ? ((cur.row0 + r) * N + col0 + 8 * half) * 2 : 0x7fff0000;
-#pragma unroll
-        for (int jj = 0; jj < TNO; ++jj) {
-#pragma unroll
-          for (int qq = 0; qq < 4; qq += 2) {
-            unsigned pk[2][2];
-#pragma unroll
-            for (int dq = 0; dq < 2; ++dq) {
-#pragma unroll
-              for (int tp = 0; tp < 2; ++tp) {  // two neighbouring columns at a time
-                const int i = (qq + dq) * 4 + tp * 2;
-                if (kDual) {
-                  // both products rounded to bf16 (one packed conversion each), then silu(g) * u on them
-                  const unsigned gb = pack_bf16x2(acc[mi][jj][i], acc[mi][jj][i + 1]);
-                  const unsigned ub = pack_bf16x2(acc[mi][jj + TN / 2][i], acc[mi][jj + TN / 2][i + 1]);
-                  if (pass == 0) {
-                    const float g0 = __uint_as_float(gb << 16), g1 = __uint_as_float(gb & 0xffff0000u);
-                    const float u0 = __uint_as_float(ub << 16), u1 = __uint_as_float(ub & 0xffff0000u);
-                    pk[dq][tp] = pack_bf16x2(silu_rcp(g0) * u0, silu_rcp(g1) * u1);
-                  } else {
-                    pk[dq][tp] = pass == 1 ? gb : ub;
-                  }
-                } else {
-                  pk[dq][tp] = pack_bf16x2(acc[mi][jj][i], acc[mi][jj][i + 1]);
-                }
-              }
-            }
-            // before: this lane has columns 8 qq + 4 half + 0..3 (pk[0]) and 8 (qq + 1) + 4 half + 0..3
-            // (pk[1]); after: columns 8 (qq + half) + 0..7
-            const auto lo = __builtin_amdgcn_permlane32_swap(pk[0][0], pk[1][0], false, false);
-            const auto hi = __builtin_amdgcn_permlane32_swap(pk[0][1], pk[1][1], false, false);
-            const u32x4_t val = {lo[0], hi[0], lo[1], hi[1]};
-            const int col = jj * 32 + 8 * qq;  // + 8 * half, already in row_off
-            const int off = col < cols_left ? row_off : 0x7fff0000;
-            // plain stores: a 128-byte line of the result is put together from four of these stores in the
-            // L2 (as non-temporal stores the 32-byte pieces cost 17 % of the down projection)
-            __builtin_amdgcn_raw_buffer_store_b128(val, out_rsrc, off + col * 2, 0, 0);
-            // keeps the compiler from computing many column runs at once (register pressure)
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        }
-      }
-    };
-    write_pass(std::integral_constant<int, 0>{});
-    if (kDual && save0 != nullptr) {
-      write_pass(std::integral_constant<int, 1>{});
-      write_pass(std::integral_constant<int, 2>{});
-    }
+    // ---- epilogue: straight from the accumulators to memory (no LDS, no barrier) ----
+    store_transposed_accumulators<Cfg>(acc, wm, wn, cur.row0, cur.rows, cur.n0, N, dense_rows, C, save0, save1);
     if (!have_next) break;
     cur = nxt;
   }

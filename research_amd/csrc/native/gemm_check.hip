@@ -15,6 +15,7 @@
 //                               every expert matrix read into the memory-side cache beforehand
 //   gemm_check time_tn_stages   the weight-gradient kernel with two, three and four operand stages
 //   gemm_check time_c2_down     the down projection with 256 x 256 against 256 x 128 tiles, caches warm and cold
+//   gemm_check time_down        the down projection's kernels at the three large configurations' shapes, caches cold
 //   gemm_check time_prio        the stream kernel with and without raised wave priority around its MFMAs
 //   (a second argument "nocheck" skips the correctness cases)
 #include "grouped_gemm_bwd.hpp"
@@ -186,7 +187,8 @@ static void launch(Problem& p, bool dense) {
                          (int)Cfg::SMEM_BYTES));
   kernel<<<(unsigned)tiles_grid, Cfg::NT, Cfg::SMEM_BYTES>>>(
       p.A, p.B0, Cfg::kDual ? p.B1 : nullptr, p.C, dense ? nullptr : p.dgs, dense ? nullptr : p.doff, p.E, p.rows,
-      p.K, p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, nullptr, nullptr);
+      p.K, p.N, (int)mt, (int)nt, p.top_k > 0 ? p.dmap : nullptr, p.top_k > 0 ? p.top_k : 1, p.a_rows, nullptr, nullptr, 0,
+      0);
 }
 
 template <typename Cfg>
@@ -483,7 +485,7 @@ static void time_backward() {
       time_launches(save ? "forward gate/up, products kept" : "forward gate/up", 4.0 * rows * H * I, 10, [&] {
         kernel<<<(unsigned)gemm_grid(mt, nt), GateUpCfg::NT, GateUpCfg::SMEM_BYTES>>>(
             p.A, p.B0, p.B1, p.C, p.dgs, p.doff, E, rows, H, I, (int)mt, (int)nt, p.dmap, topk, p.a_rows,
-            save ? s0 : nullptr, save ? s1 : nullptr);
+            save ? s0 : nullptr, save ? s1 : nullptr, 0, 0);
       });
     hipFree(s0); hipFree(s1);
     release(p);
@@ -944,46 +946,6 @@ int main(int argc, char** argv) {
     CK(hipDeviceSynchronize());
     release(g); release(d); release(sq);
   }
-  if (ok && argc > 1 && !strcmp(argv[1], "time_unequal_tn")) {
-    // weight gradients over groups of very unequal sizes (128 groups, 131072 rows)
-    const int E = 128, rows = 131072, H = 2048, I = 768;
-    Problem p = make(E, rows, H, I, 41, true, 0, 1.0f);
-    int longest = 0;
-    for (int n : p.gs) longest = std::max(longest, n);
-    printf("longest group: %d rows of %d\n", longest, rows);
-    uint16_t* D0 = random_bf16((size_t)rows * I, 42, 1.0f);
-    uint16_t* D1 = random_bf16((size_t)rows * I, 43, 1.0f);
-    uint16_t *C0, *C1;
-    CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
-    Problem q = make(E, rows, I, H, 41, true, 0, 1.0f);
-    uint16_t* dYp = random_bf16((size_t)rows * H, 44, 1.0f);
-    for (int rep = 0; rep < 3; ++rep) {
-      time_launches("wgrad gate/up, unequal groups", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
-      time_launches("wgrad down, unequal groups", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
-    }
-    hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
-    release(p); release(q);
-  }
-  if (ok && argc > 1 && !strcmp(argv[1], "time_persistent_tn")) {
-    const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
-    Problem p = make(E, rows, H, I, 21, false, 0, 1.0f);
-    uint16_t* D0 = random_bf16((size_t)rows * I, 31, 1.0f);
-    uint16_t* D1 = random_bf16((size_t)rows * I, 32, 1.0f);
-    uint16_t *C0, *C1;
-    CK(hipMalloc(&C0, (size_t)E * H * I * 2)); CK(hipMalloc(&C1, (size_t)E * H * I * 2));
-    Problem q = make(E, rows, I, H, 23, false, 0, 1.0f);
-    uint16_t* dYp = random_bf16((size_t)rows * H, 37, 1.0f);
-    for (int rep = 0; rep < 3; ++rep) {
-      g_one_tile_per_workgroup = true;
-      time_launches("wgrad gate/up, one pair per workgroup", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
-      time_launches("wgrad down, one pair per workgroup", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
-      g_one_tile_per_workgroup = false;
-      time_launches("wgrad gate/up, persistent (library)", 4.0 * rows * H * I, 10, [&] { launch_tn<WgradDualCfg>(p, D0, D1, C0, C1, false, false, false); });
-      time_launches("wgrad down, persistent (library)", 2.0 * rows * H * I, 10, [&] { launch_tn<WgradCfg>(q, dYp, nullptr, C0, nullptr, false, false, false); });
-    }
-    hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
-    release(p); release(q);
-  }
   if (ok && argc > 1 && !strcmp(argv[1], "time_tn_stages")) {
     // the weight-gradient kernel with two stages of 64 rows, and three and four (the library's) of 32
     using Dual64x2 = WgradDualGatherCfg;
@@ -1032,22 +994,6 @@ int main(int argc, char** argv) {
     hipFree(D0); hipFree(D1); hipFree(C0); hipFree(C1); hipFree(dYp);
     release(p); release(q);
   }
-  if (ok && argc > 1 && !strcmp(argv[1], "time_persistent_nt")) {
-    const int E = 64, T = 16384, topk = 8, H = 2048, I = 1408, rows = T * topk;
-    Problem p = make(E, rows, H, I, 21, false, 0, 1.0f);   // Z = dYp @ Wd^T
-    Problem q = make(E, rows, I, H, 22, false, 0, 1.0f);   // dXp = dG @ Wg^T + dU @ Wu^T
-    uint16_t* A1 = random_bf16((size_t)rows * I, 33, 1.0f);
-    for (int rep = 0; rep < 3; ++rep) {
-      g_one_tile_per_workgroup = true;
-      time_launches("dgrad down, one tile per workgroup", 2.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(p, nullptr, 1, false); });
-      time_launches("dgrad gate/up, one tile per workgroup", 4.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(q, A1, 2, false); });
-      g_one_tile_per_workgroup = false;
-      time_launches("dgrad down, persistent (library)", 2.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(p, nullptr, 1, false); });
-      time_launches("dgrad gate/up, persistent (library)", 4.0 * rows * H * I, 10, [&] { launch_nt<DgradCfg>(q, A1, 2, false); });
-    }
-    hipFree(A1);
-    release(p); release(q);
-  }
   if (ok && argc > 1 && !strcmp(argv[1], "time_persistent")) {
     Problem g = make(64, 131072, 2048, 1408, 4, false, 0, 1.0f);
     Problem d = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
@@ -1070,21 +1016,40 @@ int main(int argc, char** argv) {
     }
     release(g); release(d);
   }
-  if (ok && argc > 1 && !strcmp(argv[1], "time_stores")) {
-    // plain against non-temporal stores of the result, alternating on one problem
-    using GateUpNt = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128 + 32768>;
-    using DownPlain = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128>;
-    Problem g = make(64, 131072, 2048, 1408, 4, false, 0, 1.0f);
-    Problem d = make(64, 131072, 1408, 2048, 5, false, 0, 1.0f);
-    ok &= check<GateUpNt>("gate/up non-temporal stores", g);
-    ok &= check<DownPlain>("down plain stores", d);
-    for (int rep = 0; rep < 3; ++rep) {
-      timeit<GateUpCfg>("gate/up plain stores (library)", g, 20);
-      timeit<GateUpNt>("gate/up non-temporal stores", g, 20);
-      timeit<DownPlain>("down plain stores", d, 20);
-      timeit<DownCfg>("down non-temporal stores (library)", d, 20);
+  if (ok && argc > 1 && !strcmp(argv[1], "time_down")) {
+    // The down projection at the shapes of the three large configurations -- 44, 22 and 12 k steps of 64
+    // under a 256 x 256 result tile -- with the caches cold, as inside a layer: the library's kernel, the
+    // stream kernel (four stages of 32 and two of 64), and the library's loop with the results written
+    // straight from transposed accumulators instead of through LDS.
+    using DownDirect = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128 + 2048>;
+    {
+      Problem p = make(7, 3001, 576, 392, 71, true, 0, 1.0f);
+      ok &= check<DownDirect>("down ragged, results from accumulators", p);
+      release(p);
+      Problem u = make(40, 70000, 128, 264, 72, true, 0, 1.0f);
+      ok &= check<DownDirect>("down many tiles, results from accumulators", u);
+      release(u);
     }
-    release(g); release(d);
+    struct Shape { const char* name; int E, rows, K, N; bool skew; };
+    const Shape shapes[3] = {{"C2", 16, 16384, 2816, 1024, false}, {"C3", 64, 131072, 1408, 2048, false},
+                             {"C4", 128, 131072, 768, 2048, true}};
+    for (const Shape& sh : shapes) {
+      Problem d = make(sh.E, sh.rows, sh.K, sh.N, 5, sh.skew, 0, 1.0f);
+      char name[96];
+      for (int rep = 0; ok && rep < 3; ++rep) {
+        snprintf(name, sizeof name, "%s down, library", sh.name);
+        timeit_cold<DownCfg>(name, d, 20);
+        g_stream = true;
+        snprintf(name, sizeof name, "%s down, stream 4 x 32", sh.name);
+        timeit_cold<DownStreamCfg>(name, d, 20);
+        snprintf(name, sizeof name, "%s down, stream 2 x 64", sh.name);
+        timeit_cold<DownStream2Cfg>(name, d, 20);
+        g_stream = false;
+        snprintf(name, sizeof name, "%s down, results from accumulators", sh.name);
+        timeit_cold<DownDirect>(name, d, 20);
+      }
+      release(d);
+    }
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_backward")) time_backward();
   if (ok && argc > 1 && !strcmp(argv[1], "time_decode")) time_decode();

@@ -20,7 +20,6 @@ namespace {
 
 // A workgroup of NW waves routes 16*NW tokens with 64*NW threads (4 lanes per token in the
 // selection phase).
-constexpr float kFixedScale = kImportanceScale;  // importance is summed in 32.32 fixed point
 
 // ---- fully specified fp32 sigmoid ------------------------------------------
 __device__ __forceinline__ float exp_fixed(float x) {
@@ -48,6 +47,7 @@ __device__ __forceinline__ float exp_fixed(float x) {
 
 __device__ __forceinline__ float sigmoid_fixed(float z) {
 #pragma clang fp contract(off)
+  if (z != z) return z;  // fmaxf / fminf below would turn a NaN into a finite score
   float t = -z;
   t = fmaxf(t, -86.0f);
   t = fminf(t, 86.0f);
@@ -130,14 +130,17 @@ __device__ __forceinline__ float quad_xor_f32(float v) {
   return __builtin_bit_cast(float, quad_xor_i32<kXor>(__builtin_bit_cast(int, v)));
 }
 
-// Order-preserving map of a non-NaN float onto a signed integer: a > b as floats <=> key(a) > key(b)
-// (-0 is canonicalised to +0 first, so equal floats have equal keys).  No float maps to INT_MIN,
-// which therefore serves as "already taken".
+// Order-preserving map of a float onto a signed integer: a > b as floats <=> key(a) > key(b)
+// (-0 is canonicalised to +0 first, so equal floats have equal keys).  Every NaN gets one key below
+// -infinity's: a NaN score is chosen last, among NaNs the lower index first -- the order a stable
+// descending sort gives (NumPy sorts NaN to the end), and one that keeps the chosen index in range.
+// No float maps to INT_MIN, which therefore serves as "already taken".
+constexpr int kTakenKey = (int)0x80000000u;
+constexpr int kNanKey = kTakenKey + 1;
 __device__ __forceinline__ int order_key(float v) {
   const int bits = __builtin_bit_cast(int, v + 0.0f);
-  return bits ^ ((bits >> 31) & 0x7fffffff);
+  return v != v ? kNanKey : bits ^ ((bits >> 31) & 0x7fffffff);
 }
-constexpr int kTakenKey = (int)0x80000000u;
 
 // K rounds of "largest remaining score + bias, lower index on ties" for one token, by its four
 // lanes: lane q owns experts [e_begin, e_begin + EQ) and keeps their keys in registers; a taken
@@ -186,21 +189,21 @@ __device__ __forceinline__ void select_from_registers(const RouterSmem& sm, cons
   }
 }
 
-// The same selection for any expert count: the lane re-reads its quarter from LDS in every round.
+// The same selection (same keys, same comparisons) for any expert count: the lane re-reads its quarter
+// from LDS in every round.
 __device__ __forceinline__ void select_from_lds(const RouterSmem& sm, const float* row, int e_begin, int eq, int E,
                                                 bool row_ok, int t, int q, int K) {
 #pragma clang fp contract(off)
   unsigned long long taken = 0ull;
   for (int r = 0; r < K; ++r) {
-    float best_v = 0.0f;
-    int best_e = -1;
+    int best_k = kTakenKey, best_e = -1;
     if (row_ok) {
       for (int j = 0; j < eq; ++j) {
         const int e = e_begin + j;
         if (e < E && !((taken >> j) & 1ull)) {
-          const float v = row[e] + sm.bias[e];
-          if (best_e < 0 || v > best_v) {
-            best_v = v;
+          const int k = order_key(row[e] + sm.bias[e]);
+          if (k > best_k) {  // strictly: the lower index keeps a tie
+            best_k = k;
             best_e = e;
           }
         }
@@ -208,11 +211,11 @@ __device__ __forceinline__ void select_from_lds(const RouterSmem& sm, const floa
     }
 #pragma unroll
     for (int m = 1; m <= 2; m <<= 1) {
-      const float ov = __shfl_xor(best_v, m, 4);
+      const int ok = __shfl_xor(best_k, m, 4);
       const int oe = __shfl_xor(best_e, m, 4);
-      const bool take = oe >= 0 && (best_e < 0 || ov > best_v || (ov == best_v && oe < best_e));
+      const bool take = oe >= 0 && (best_e < 0 || ok > best_k || (ok == best_k && oe < best_e));
       if (take) {
-        best_v = ov;
+        best_k = ok;
         best_e = oe;
       }
     }
@@ -331,7 +334,7 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
       ids_out[o] = e;
       Elem<T>::store(weights_out + o, w);
       atomicAdd(&sm.cnt[e], 1);
-      atomicAdd(&sm.imp[e], (unsigned long long)(w * kFixedScale));
+      atomicAdd(&sm.imp[e], importance_term(w));
     }
   }
   __syncthreads();
@@ -795,6 +798,11 @@ struct LayerPlan {
   int32_t* inverse;
   bool stats_done;
   bool plan_done;
+  // the call runs beside a launch that fills the CUs (the decode path's gate/up): the finishing
+  // workgroup then takes its 64-token form where that holds the batch -- 256 threads and a fifth of
+  // the LDS, which a CU can place next to three resident GEMM workgroups; the 1024-thread form would
+  // wait for a CU to drain
+  bool beside_gemm;
 };
 
 template <typename T, bool kFromLogits>
@@ -820,7 +828,9 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
         return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
       // Two launches when one workgroup can hold the epilogue of the whole call: partial sums over
       // k slices from many workgroups, then the finishing workgroup.
-      const int finish_tok = router_smem_bytes((int)E, (int)K, 256) <= 160 * 1024 ? 256 : 64;
+      const int finish_tok = (layer != nullptr && layer->beside_gemm && tokens <= 64)                  ? 64
+                             : router_smem_bytes((int)E, (int)K, 256) <= 160 * 1024 ? 256
+                                                                                    : 64;
       if (tokens > 0 && tokens <= finish_tok && router_smem_bytes((int)E, (int)K, finish_tok) <= 160 * 1024) {
         const int slice_rows = router_slice_rows((int)H);
         const int slices = (int)((H + slice_rows - 1) / slice_rows);
@@ -960,7 +970,7 @@ int router_for_layer(const void* x, const void* w_router, const float* expert_bi
                      int64_t K, double route_scale, int dtype, int32_t* expert_ids, void* weights, float* scores,
                      float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
                      int32_t* source_order, int32_t* inverse, void* workspace, size_t workspace_bytes,
-                     int score_func, bool* stats_done, bool* plan_done, hipStream_t s) {
+                     int score_func, bool* stats_done, bool* plan_done, hipStream_t s, bool beside_gemm) {
   int rc = validate_router(T, H, E, K, route_scale, dtype, true);
   if (rc) return rc;
   JT_REQUIRE(score_func_ok(score_func), "router: unknown score function %d", score_func);
@@ -969,7 +979,7 @@ int router_for_layer(const void* x, const void* w_router, const float* expert_bi
   JT_REQUIRE(group_sizes && offsets && (T == 0 || (source_order && inverse)), "router: null pointer argument");
   if (workspace_bytes < jtmoe_router_workspace_bytes(E))
     return fail(JTMOE_EWORKSPACE, "router: workspace %zu < %zu bytes", workspace_bytes, jtmoe_router_workspace_bytes(E));
-  LayerPlan layer{group_sizes, offsets, source_order, inverse, false, false};
+  LayerPlan layer{group_sizes, offsets, source_order, inverse, false, false, beside_gemm};
   if (dtype == JTMOE_BF16)
     rc = launch_router<bf16_raw, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
                                         scores, expert_counts, importance, nullptr, workspace, s, score_func, &layer);

@@ -40,10 +40,18 @@ def test_workspace_sizing_is_pure_host_arithmetic():
     T, H, E, K, I, Is = 16384, 2048, 64, 8, 1408, 2816
     total = lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, _ffi.JTMOE_BF16)
     A = T * K
-    payload = 2 * (A * H + A * I + A * H + T * Is + T * H)
+    # bf16 at these sizes: the grouped GEMM gathers its rows through the permutation, so the workspace
+    # holds the activation, the expert outputs and the shared experts' buffers, but no permuted copy of x
+    assert lib.jtmoe_grouped_swiglu_gather_supported(T, H, I, _ffi.JTMOE_BF16) == 1
+    payload = 2 * (A * I + A * H + T * Is + T * H)
     assert payload <= total <= payload + 2**21  # + metadata, alignment and the router's partial sums (0.5 MiB at E=64)
+    assert total < 1.14e9  # 1.67e9 with the permuted copy
     assert total % 256 == 0
-    assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, _ffi.JTMOE_F32) >= 2 * payload
+    # fp32 (and any shape the gathering GEMM does not take, e.g. H not a multiple of 64) keeps the copy
+    assert lib.jtmoe_grouped_swiglu_gather_supported(T, H, I, _ffi.JTMOE_F32) == 0
+    assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, _ffi.JTMOE_F32) >= 2 * (payload + 2 * A * H)
+    odd = lib.jtmoe_workspace_bytes(T, H + 8, E, K, I, Is, _ffi.JTMOE_BF16)
+    assert odd >= 2 * (A * (H + 8) + A * I + A * (H + 8) + T * Is + T * (H + 8))
     assert lib.jtmoe_workspace_bytes(0, H, E, K, I, 0, _ffi.JTMOE_BF16) > 0
     assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, 7) == 0  # unknown dtype
     assert lib.jtmoe_router_workspace_bytes(E) >= 12 * E

@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import json
 
+import numpy as np
 import pytest
 import torch
 
@@ -32,7 +33,7 @@ def test_benchmark_of_the_decode_shape_writes_its_artifact(tmp_path):
     assert row["same_routing_fraction"] >= 0.95, row
     assert row["max_abs_error_over_max_abs"] <= 2e-2, row  # the stated bf16 tolerance
     assert row["jtmoe_ms"]["min"] > 0 and row["jtmoe_ms"]["min"] <= row["jtmoe_ms"]["p50"] <= row["jtmoe_ms"]["max"]
-    assert row["speedup_p50"] > 0.0, row  # reported, not asserted on: a timing ratio is no correctness property
+    assert np.isfinite(row["speedup_p50"])  # a reported figure: a timing ratio is no correctness property
     stored = json.loads((tmp_path / "diagnostics" / "kernel_benchmarks" / "moe.json").read_text())
     assert stored["rows"][0]["config"] == "C5" and stored["artifact_path"] == payload["artifact_path"]
     assert "C5 (bfloat16)" in kernel_bench.format_moe_benchmark(payload)

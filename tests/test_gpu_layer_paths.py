@@ -121,3 +121,72 @@ def check_random_layer_shapes(gpu, seed: int, cases: int) -> None:
         assert np.array_equal(host(plan.source_order), d.source_order), tag
         assert np.array_equal(host(plan.group_sizes), d.group_sizes), tag
         assert bool(torch.isfinite(layer.y.float()).all()), tag
+
+
+# (tokens, hidden, experts, top_k, d_ff, shared width): at most 64 tokens, tokens * top_k >= 2 * experts
+DECODE_CASES = [
+    (64, 2048, 64, 8, 1408, 0),   # the decode shape of the benchmark
+    (64, 2048, 64, 8, 128, 256),  # with shared experts
+    (16, 256, 64, 8, 64, 0),      # tokens * top_k = 2 * experts: the smallest batch that takes the path
+    (40, 128, 16, 2, 192, 0),
+    (33, 192, 8, 8, 64, 64),      # every token picks every expert
+    (15, 256, 64, 8, 64, 0),      # one token short: the ordinary path (the comparison must hold either way)
+]
+
+
+@pytest.mark.parametrize("tokens,hidden,experts,top_k,d_ff,shared_width", DECODE_CASES)
+def test_decode_path_equals_the_stand_alone_operators(gpu, tokens, hidden, experts, top_k, d_ff, shared_width):
+    """At decode-sized batches the layer runs every token through every expert beside the router (on a
+    second stream) and the down projection picks the routed rows.  The output must equal, bit for bit,
+    router -> dispatch -> gathering grouped SwiGLU -> combine called one by one, twice in a row, and
+    through a workspace that a larger call has used in between."""
+    rng = np.random.default_rng(tokens * 131 + experts)
+    x = dev(rng.standard_normal((tokens, hidden)).astype(np.float32), gpu, "bf16")
+    w_router = dev((rng.standard_normal((hidden, experts)) * 0.1).astype(np.float32), gpu, "bf16")
+    gate = dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, "bf16")
+    up = dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, "bf16")
+    down = dev((rng.standard_normal((experts, d_ff, hidden)) * 0.05).astype(np.float32), gpu, "bf16")
+    shared = None
+    if shared_width:
+        shared = tuple(dev((rng.standard_normal(s) * 0.05).astype(np.float32), gpu, "bf16")
+                       for s in ((hidden, shared_width), (hidden, shared_width), (shared_width, hidden)))
+
+    route = ops.router(x, w_router, None, top_k, 1.0)
+    plan = ops.dispatch(route.expert_ids, experts)
+    packed_y = ops.grouped_swiglu_gather(x, plan.source_order, top_k, gate, up, down, plan.group_sizes, plan.offsets)
+    want = ops.combine(packed_y, plan.inverse, route.weights, None if shared is None else ops.shared_swiglu(x, *shared))
+
+    first = ops.moe_forward(x, w_router, None, gate, up, down, top_k, 1.0, shared=shared)
+    assert torch.equal(first.y, want)
+    assert torch.equal(first.source_order, plan.source_order) and torch.equal(first.expert_ids, route.expert_ids)
+    big = dev(rng.standard_normal((300, hidden)).astype(np.float32), gpu, "bf16")
+    ops.moe_forward(big, w_router, None, gate, up, down, top_k, 1.0, shared=shared)  # other rows through the same workspace
+    again = ops.moe_forward(x, w_router, None, gate, up, down, top_k, 1.0, shared=shared)
+    assert torch.equal(again.y, want)
+    torch.cuda.synchronize()
+
+
+def test_decode_path_follows_work_on_the_callers_stream(gpu):
+    """The second stream starts only when the caller's stream has reached the call (its input may still
+    be being written there) and the caller's stream continues only when the second stream is done."""
+    rng = np.random.default_rng(77)
+    T, H, E, K, I = 64, 512, 64, 8, 128
+    w_router = dev((rng.standard_normal((H, E)) * 0.1).astype(np.float32), gpu, "bf16")
+    gate = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    up = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    down = dev((rng.standard_normal((E, I, H)) * 0.05).astype(np.float32), gpu, "bf16")
+    base = dev(rng.standard_normal((T, H)).astype(np.float32), gpu, "bf16")
+    want = ops.moe_forward((base.float() * 2).to(torch.bfloat16), w_router, None, gate, up, down, K, 1.0).y.clone()
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream(device=gpu)
+    stream.wait_stream(torch.cuda.current_stream(gpu))
+    with torch.cuda.stream(stream):
+        for _ in range(5):
+            filler = torch.randn((4096, 4096), device=gpu) @ torch.randn((4096, 4096), device=gpu)  # keeps the stream busy
+            x = (base.float() * 2).to(torch.bfloat16)  # written on this stream right before the call
+            y = ops.moe_forward(x, w_router, None, gate, up, down, K, 1.0).y
+            doubled = y.float() * 2  # read on this stream right after the call
+            assert torch.equal(doubled, want.float() * 2)
+            del filler
+    torch.cuda.current_stream(gpu).wait_stream(stream)
+    torch.cuda.synchronize()

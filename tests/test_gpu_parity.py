@@ -112,6 +112,33 @@ def test_routing_decision_with_negative_zero_and_infinite_biased_scores(gpu, exp
     assert not np.any(np.isin(host(got.expert_ids), [1, 6]))
 
 
+@pytest.mark.parametrize("experts,top_k", [(64, 8), (24, 3), (16, 16), (5, 5)])
+def test_routing_decision_with_nan_logits_stays_in_range_and_orders_nan_last(gpu, experts, top_k):
+    """What lax.top_k does with NaN is not pinned by any reference test.  Here a NaN logit gives a NaN
+    score, which is chosen after every number (-inf included) and, among NaNs, lower index first -- the
+    order of a stable descending sort, which is also the oracle's -- so that ids stay inside [0, E) and the
+    selection kernels for the usual expert counts and for the others agree."""
+    rng = np.random.default_rng(experts)
+    tokens = 96
+    logits = O.bf16_round((rng.standard_normal((tokens, experts)) * 2.0).astype(np.float32))
+    logits[0, :] = np.nan                       # nothing but NaN: ids 0 .. K-1
+    logits[1, ::2] = np.nan                     # half of the row
+    logits[2, 0] = np.nan
+    logits[3, : experts - 1] = np.nan           # one number left: it comes first
+    logits[4, 1] = -np.inf                      # -inf is still chosen before a NaN
+    logits[4, 2] = np.nan
+    with np.errstate(invalid="ignore"):
+        want = O.router_from_logits(logits, None, top_k, 1.0, "bf16")
+    got = ops.router_from_logits(dev(logits, gpu), None, top_k, 1.0, dtype=torch.bfloat16)
+    ids = host(got.expert_ids)
+    assert ids.min() >= 0 and ids.max() < experts
+    assert np.array_equal(ids, want.expert_ids)
+    assert np.array_equal(host(got.scores), want.scores, equal_nan=True)
+    assert np.array_equal(host(got.weights), want.weights, equal_nan=True)
+    assert np.array_equal(host(got.expert_counts), np.bincount(ids.reshape(-1), minlength=experts).astype(np.float32))
+    assert np.all(np.isfinite(host(got.importance)))  # a NaN weight adds nothing
+
+
 @pytest.mark.parametrize("case", ["router_order", "router_bias_scale"])
 def test_router_known_answers(gpu, kat, case):
     c = kat[case]
