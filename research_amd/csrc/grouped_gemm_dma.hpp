@@ -128,6 +128,9 @@ struct DmaGemmCfg {
   static constexpr size_t PIPE_BYTES = (size_t)NSTAGE * STAGE_BYTES;
   static constexpr size_t SMEM_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
   static constexpr int GROUP_M = 4;
+  // A four-wave workgroup whose waves hold 128 accumulators each is meant to share its CU with a second
+  // one (two waves per SIMD): the register allocation is held to half of the file.
+  static constexpr int MIN_WAVES_PER_EU = (NT == 256 && TM * TN * 16 >= 128) ? 2 : 1;
   static_assert(BNE % 128 == 0, "B tile is made of 128-column sub-tiles");
   static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
   static_assert((BM * CPRA) % NT == 0 && (BK * 16) % NT == 0, "tile must divide evenly over the threads");
@@ -228,7 +231,7 @@ __device__ __forceinline__ void store_transposed_accumulators(const f32x16_t (&a
 }
 
 template <typename Cfg>
-__global__ __launch_bounds__(Cfg::NT) void grouped_gemm_dma_kernel(
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::MIN_WAVES_PER_EU))) void grouped_gemm_dma_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
     uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
     int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,

@@ -1022,9 +1022,19 @@ int main(int argc, char** argv) {
     // stream kernel (four stages of 32 and two of 64), and the library's loop with the results written
     // straight from transposed accumulators instead of through LDS.
     using DownDirect = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 64 + 128 + 2048>;
+    // Half-size tiles in workgroups of four waves, two workgroups to a CU (each SIMD then holds waves of two
+    // tiles that are in different phases: one tile's epilogue and first loads run under the other's MFMAs)
+    using Down256x128w4 = DmaGemmCfg<256, 128, 32, 4, 1, false, 2, 16 + 128 + 32768>;
+    using Down256x128w4s3 = DmaGemmCfg<256, 128, 32, 4, 1, false, 3, 16 + 128 + 32768>;
+    using Down128x256w4 = DmaGemmCfg<128, 256, 32, 2, 2, false, 2, 16 + 128 + 32768>;
+    using Down128x256w4s3 = DmaGemmCfg<128, 256, 32, 2, 2, false, 3, 16 + 128 + 32768>;
     {
       Problem p = make(7, 3001, 576, 392, 71, true, 0, 1.0f);
       ok &= check<DownDirect>("down ragged, results from accumulators", p);
+      ok &= check<Down256x128w4>("down ragged, 256 x 128, four waves", p);
+      ok &= check<Down256x128w4s3>("down ragged, 256 x 128, four waves, 3 stages", p);
+      ok &= check<Down128x256w4>("down ragged, 128 x 256, four waves", p);
+      ok &= check<Down128x256w4s3>("down ragged, 128 x 256, four waves, 3 stages", p);
       release(p);
       Problem u = make(40, 70000, 128, 264, 72, true, 0, 1.0f);
       ok &= check<DownDirect>("down many tiles, results from accumulators", u);
@@ -1047,6 +1057,14 @@ int main(int argc, char** argv) {
         g_stream = false;
         snprintf(name, sizeof name, "%s down, results from accumulators", sh.name);
         timeit_cold<DownDirect>(name, d, 20);
+        snprintf(name, sizeof name, "%s down, 256 x 128 x 32, 4 waves, 2 per CU", sh.name);
+        timeit_cold<Down256x128w4>(name, d, 20);
+        snprintf(name, sizeof name, "%s down, 256 x 128 x 32, 4 waves, 3 stages", sh.name);
+        timeit_cold<Down256x128w4s3>(name, d, 20);
+        snprintf(name, sizeof name, "%s down, 128 x 256 x 32, 4 waves, 2 per CU", sh.name);
+        timeit_cold<Down128x256w4>(name, d, 20);
+        snprintf(name, sizeof name, "%s down, 128 x 256 x 32, 4 waves, 3 stages", sh.name);
+        timeit_cold<Down128x256w4s3>(name, d, 20);
       }
       release(d);
     }
