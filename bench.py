@@ -83,13 +83,14 @@ def cpu_baseline(name: str, sample_tokens: int | None) -> dict:
     args = (inp["x"], inp["w_router"], inp["expert_bias"], inp["gate"], inp["up"], inp["down"])
     small = inp["x"][:, : min(64, sample_tokens)]
     O.moe_forward(small, *args[1:], **kwargs)  # first call excluded
-    # whole calls until at least two seconds of host work have been timed (one call at the large shapes)
+    # whole calls until at least two seconds of host work have been timed, and never fewer than two calls
+    # (at the large shapes a call takes several seconds: two of them, the mean reported)
     calls, t0 = 0, time.perf_counter()
     while True:
         out = O.moe_forward(*args, **kwargs)
         calls += 1
         total = time.perf_counter() - t0
-        if total >= 2.0 or calls >= 200:
+        if (total >= 2.0 and calls >= 2) or calls >= 200:
             break
     dt = total / calls
     assert np.isfinite(out.y).all()
@@ -210,8 +211,11 @@ def train_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, work) -> dic
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=50)
-    parser.add_argument("--warmup", type=int, default=20)
+    # defaults: 50 timed steps after 20 untimed ones at the large configurations (C3: 54 + 135 ms of load);
+    # the small ones get as many as keep the chip under load for about as long before and while timing
+    # (its clocks need some tens of milliseconds to settle): C2 150 + 400, C5 300 + 800, C1 300 + 800
+    parser.add_argument("--steps", type=int, default=None)
+    parser.add_argument("--warmup", type=int, default=None)
     parser.add_argument("--config", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
     parser.add_argument("--cpu-sample-tokens", type=int, default=16384,
                         help="tokens of the workload the CPU baseline runs (the whole of C3 takes about 9 s of host work)")
@@ -219,6 +223,11 @@ def main() -> int:
     parser.add_argument("--no-train", action="store_true", help="skip the forward+backward timing")
     parser.add_argument("--no-block", action="store_true", help="skip the decoder-block and graph-replay timings")
     args = parser.parse_args()
+    default_warmup, default_steps = {"C2": (150, 400), "C5": (300, 800), "C1": (300, 800)}.get(args.config, (20, 50))
+    if args.steps is None:
+        args.steps = default_steps
+    if args.warmup is None:
+        args.warmup = default_warmup
     if args.gpus != 1:
         print(f"bench.py measures one GPU: the layer runs with every expert local and no collective; "
               f"--gpus {args.gpus} is not supported in this build", file=sys.stderr)
@@ -418,6 +427,12 @@ def main() -> int:
         "roofline": roofline,
         "stages": stages,
     }
+    if lib.jtmoe_moe_forward_uses_second_stream(T, cfg["H"], cfg["E"], cfg["K"], cfg["I"], code):
+        # ms_per_step is the call as a caller runs it; the stage times come from the timed variant of the
+        # call, which keeps every launch on one stream so that a stage's time is its kernels' time
+        line["stages"]["note"] = ("decode path: in the timed step the gate/up launch (every token through every "
+                                  "expert) runs on the caller's stream beside the router and the plan on a second "
+                                  "one; the stage times are taken with all launches on one stream")
     if not args.no_block:
         if T <= 2048:
             line["graph_replay"] = graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, max(args.steps, 50))

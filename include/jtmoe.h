@@ -265,7 +265,19 @@ int jtmoe_smebu_update(const float* router_counts, float* momentum, float* exper
  *        GEMM fetches its rows through the permutation, the workspace holds no
  *        permuted copy of x ([A,H]: a third of it at 64 experts, top-8, H = 2048),
  *        and x, gate, up and down must be 16-byte aligned (JTMOE_EINVAL otherwise).
+ *   streams: everything is enqueued on `stream`, with one exception.  Where
+ *        jtmoe_moe_forward_uses_second_stream(T, H, E, K, I, dtype) holds (bf16, at most
+ *        64 tokens, T*K >= 2*E: a decode step), the gate/up launch runs every token
+ *        through every expert -- which needs nothing of the routing -- on `stream`,
+ *        and the router and the dispatch plan run beside it on a second stream of
+ *        default priority that the library creates once per device: forked from
+ *        `stream` by an event at entry and joined back by an event before the down
+ *        launch, so the call is ordered on `stream` like any other and can be
+ *        captured into a graph (the events become edges).  Results are bit for bit
+ *        those of the one-stream path.  No counterpart in the reference (XLA
+ *        schedules its own streams).
  */
+int jtmoe_moe_forward_uses_second_stream(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype);
 size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype);
 int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_bias,
                       const void* gate, const void* up, const void* down,

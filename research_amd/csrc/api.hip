@@ -455,6 +455,11 @@ extern "C" int jtmoe_smebu_update(const float* router_counts, float* momentum, f
   return check_launch("smebu_update");
 }
 
+extern "C" int jtmoe_moe_forward_uses_second_stream(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype) {
+  if (T < 0 || H <= 0 || E <= 0 || K <= 0 || I <= 0 || !dtype_ok(dtype)) return 0;
+  return decode_dense_supported(T, H, E, K, I, dtype) ? 1 : 0;
+}
+
 extern "C" size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is,
                                         int dtype) {
   if (T < 0 || H <= 0 || E <= 0 || K <= 0 || I <= 0 || Is < 0 || !dtype_ok(dtype)) return 0;

@@ -67,8 +67,8 @@ __device__ __forceinline__ void stream_gemm_body(
   static_assert(kNT || (Cfg::OPT & 128) != 0, "weight tiles in 4 x 64 blocks");
   static_assert(!kNT || !kDual, "the transposed-B form has one output per tile");
   static_assert(!kNT || (BN * CPRA) % NT == 0, "the B tile must divide evenly over the threads");
-  // Timing experiments of the stand-alone check (wrong results by construction, never launched by the
-  // library): OPT & 256 leaves out the operand loads of the steady part of the k loop, OPT & 512 its
+  // Timing experiments of the stand-alone check's time_ablation mode, which bounds what any schedule of
+  // this loop can reach (wrong results by construction, never launched by the library): OPT & 256 leaves out the operand loads of the steady part of the k loop, OPT & 512 its
   // fragment reads (the MFMAs then run on the fragments read once before the loop).
   // OPT & 1024 makes every load of the steady part fetch the tile's first k step again (operands that
   // are in the nearest cache: the cost of issuing the loads without the memory system behind them).
@@ -440,13 +440,15 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_gemm_stream_nt_kernel(
 // (alternating in one process): 1.306 ms against 1.400-1.409 ms for grouped_gemm_dma_persistent_kernel
 // and 1.315-1.320 ms for 64-deep steps with two stages.
 using GateUpStreamCfg = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128>;
-// Variants kept for the stand-alone check and its timings: 64-deep steps with two stages, and the
-// down projection's tile (0.725-0.737 ms against 0.723-0.727 ms for grouped_gemm_dma_persistent_kernel,
-// which the library keeps for that launch).
+// Variants kept for the stand-alone check and its timings (time_stream, time_down): 64-deep steps with
+// two stages, and the down projection's tile (within 2 % of grouped_gemm_dma_persistent_kernel, which
+// the library keeps for that launch, at 12, 22 and 44 k steps per tile).
 using GateUpStream2Cfg = DmaGemmCfg<256, 128, 64, 4, 2, true, 2, 16 + 128>;
 using DownStreamCfg = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128 + 32768>;
 using DownStream2Cfg = DmaGemmCfg<256, 256, 64, 2, 4, false, 2, 16 + 128 + 32768>;
 // The data-gradient products of the backward pass (transposed-B form): 256 x 256 tiles, 2 x 4 waves.
+// Checked and timed by the stand-alone check (time_stream_nt) against grouped_gemm_nt_kernel, which
+// the library launches: the transposed-B form measures equal or slower there.
 using DgradStreamCfg = DmaGemmCfg<256, 256, 32, 2, 4, false, 4, 16 + 128>;
 
 }  // namespace jtmoe
