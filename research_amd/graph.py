@@ -1,13 +1,15 @@
 """Replay of the layer from a captured HIP graph, for callers whose per-call host cost matters.
 
-At 64 tokens the kernels of one layer call take about 0.22 ms.  The library's own host side adds
+At 64 tokens the kernels of one layer call take about 0.19 ms.  The library's own host side adds
 about 0.05 ms per call, hidden behind the GPU when calls are issued back to back; a caller with a
 heavier host side (more Python between calls, a blocking wait after each) can capture the call
 once and replay the same kernels with a single launch.  The reference gets the equivalent from
 ``jax.jit`` (its decode step, blocks.py:262-290, runs inside one compiled program).
 
 The library's forward path only enqueues kernels (no allocation, no memset, no synchronisation),
-so it can be captured as it is.  Shapes are fixed at capture; the caller copies new inputs into
+so it can be captured as it is -- also at decode sizes, where the call forks part of its work onto a
+second stream and joins it again with events: the second stream joins the capture and the events
+become edges of the graph.  Shapes are fixed at capture; the caller copies new inputs into
 ``x`` (and may update the parameters in place) and calls ``replay()``.
 """
 
