@@ -106,7 +106,7 @@ struct DmaGemmCfg {
   // scheduling options: 16 = request the fragments of MFMA step kk+1 before issuing step kk,
   // 32 = raise the wave priority around the MFMA burst, 64 = ask the scheduler to interleave
   // one MFMA with up to three LDS reads, 128 = B tiles in 4 x 64 blocks, 2048 = (persistent kernel) results written
-  // straight from transposed accumulators instead of through LDS, 4096 = non-temporal loads of B, 32768 = non-temporal stores of the result
+  // straight from transposed accumulators instead of through LDS, 4096 = non-temporal loads of B, 8192 / 16384 = 8 / 2 m-tiles per group of the tile order instead of 4, 32768 = non-temporal stores of the result
   static constexpr int OPT = OPT_;
   static constexpr bool kDual = kDual_;
   static constexpr int BNE = kDual ? 2 * BN : BN;  // columns of the B tile in LDS
@@ -127,7 +127,9 @@ struct DmaGemmCfg {
   static constexpr size_t EPI_BYTES = (size_t)WAVES_M * WAVES_N * WM * CS * 2;
   static constexpr size_t PIPE_BYTES = (size_t)NSTAGE * STAGE_BYTES;
   static constexpr size_t SMEM_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
-  static constexpr int GROUP_M = 4;
+  // m-tiles per group of the tile order (a group = GROUP_M m-tiles x all n-tiles, walked n-tile by n-tile);
+  // option bits 8192 / 16384 select 8 / 2 for the stand-alone check's comparison of schedules
+  static constexpr int GROUP_M = (OPT_ & 8192) ? 8 : ((OPT_ & 16384) ? 2 : 4);
   // A four-wave workgroup whose waves hold 128 accumulators each is meant to share its CU with a second
   // one (two waves per SIMD): the register allocation is held to half of the file.
   static constexpr int MIN_WAVES_PER_EU = (NT == 256 && TM * TN * 16 >= 128) ? 2 : 1;

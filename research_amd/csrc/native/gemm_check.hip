@@ -15,6 +15,8 @@
 //                               every expert matrix read into the memory-side cache beforehand
 //   gemm_check time_tn_stages   the weight-gradient kernel with two, three and four operand stages
 //   gemm_check time_c2_down     the down projection with 256 x 256 against 256 x 128 tiles, caches warm and cold
+//   gemm_check time_chunks / counters_chunks   the stream kernel's gate/up launch with its tiles cut into workgroups
+//                               of 1, 2, 4, 8 tiles or one per CU, and tile-order groups of 2, 4, 8 m-tiles
 //   gemm_check time_down        the down projection's kernels at the three large configurations' shapes, caches cold
 //   gemm_check time_prio        the stream kernel with and without raised wave priority around its MFMAs
 //   (a second argument "nocheck" skips the correctness cases)
@@ -1068,6 +1070,42 @@ int main(int argc, char** argv) {
       }
       release(d);
     }
+  }
+  if (ok && argc > 1 && (!strcmp(argv[1], "time_chunks") || !strcmp(argv[1], "counters_chunks"))) {
+    // The routed gate/up launch of the third configuration with the stream kernel, its tiles cut into
+    // workgroups of 1, 2, 4 (the library's), 8 tiles or one workgroup per CU for the whole launch (0), and,
+    // at 4 tiles per workgroup, the tile order walked in groups of 2, 4 (the library's) or 8 m-tiles.
+    // time_chunks: events around 20 launches, three rounds, alternating.  counters_chunks: 12 launches of
+    // each for a hardware-counter or kernel-trace run (the variants differ in grid size or kernel name).
+    using Group8 = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 8192>;
+    using Group2 = DmaGemmCfg<256, 128, 32, 4, 2, true, 4, 16 + 128 + 16384>;
+    const bool timing = !strcmp(argv[1], "time_chunks");
+    Problem g = make(64, 131072, 2048, 1408, 4, false, 8, 1.0f);
+    g_stream = true;
+    if (timing) {
+      ok &= check<Group8>("stream gate/up, groups of 8 m-tiles", g);
+      ok &= check<Group2>("stream gate/up, groups of 2 m-tiles", g);
+    }
+    for (int rep = 0; ok && rep < (timing ? 3 : 12); ++rep) {
+      for (int chunk : {0, 1, 2, 4, 8}) {
+        g_chunk = chunk;
+        char name[80];
+        snprintf(name, sizeof name, "gate/up stream, %d tiles per workgroup", chunk);
+        if (timing) timeit<GateUpStreamCfg>(name, g, 20); else launch<GateUpStreamCfg>(g, false);
+      }
+      g_chunk = 4;
+      if (timing) {
+        timeit<Group2>("gate/up stream, 4 tiles per workgroup, groups of 2 m-tiles", g, 20);
+        timeit<Group8>("gate/up stream, 4 tiles per workgroup, groups of 8 m-tiles", g, 20);
+      } else {
+        launch<Group2>(g, false);
+        launch<Group8>(g, false);
+      }
+    }
+    CK(hipDeviceSynchronize());
+    g_chunk = -1;
+    g_stream = false;
+    release(g);
   }
   if (ok && argc > 1 && !strcmp(argv[1], "time_backward")) time_backward();
   if (ok && argc > 1 && !strcmp(argv[1], "time_decode")) time_decode();
