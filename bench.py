@@ -427,12 +427,9 @@ def main() -> int:
         "roofline": roofline,
         "stages": stages,
     }
-    if lib.jtmoe_moe_forward_uses_second_stream(T, cfg["H"], cfg["E"], cfg["K"], cfg["I"], code):
-        # ms_per_step is the call as a caller runs it; the stage times come from the timed variant of the
-        # call, which keeps every launch on one stream so that a stage's time is its kernels' time
-        line["stages"]["note"] = ("decode path: in the timed step the gate/up launch (every token through every "
-                                  "expert) runs on the caller's stream beside the router and the plan on a second "
-                                  "one; the stage times are taken with all launches on one stream")
+    if lib.jtmoe_moe_forward_takes_decode_path(T, cfg["H"], cfg["E"], cfg["K"], cfg["I"], code):
+        line["stages"]["note"] = ("decode path: the gate/up stage is one launch that runs every token through every "
+                                  "expert and holds the router and the dispatch plan in a few of its workgroups")
     if not args.no_block:
         if T <= 2048:
             line["graph_replay"] = graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, max(args.steps, 50))

@@ -265,19 +265,19 @@ int jtmoe_smebu_update(const float* router_counts, float* momentum, float* exper
  *        GEMM fetches its rows through the permutation, the workspace holds no
  *        permuted copy of x ([A,H]: a third of it at 64 experts, top-8, H = 2048),
  *        and x, gate, up and down must be 16-byte aligned (JTMOE_EINVAL otherwise).
- *   streams: everything is enqueued on `stream`, with one exception.  Where
- *        jtmoe_moe_forward_uses_second_stream(T, H, E, K, I, dtype) holds (bf16, at most
- *        64 tokens, T*K >= 2*E: a decode step), the gate/up launch runs every token
- *        through every expert -- which needs nothing of the routing -- on `stream`,
- *        and the router and the dispatch plan run beside it on a second stream of
- *        default priority that the library creates once per device: forked from
- *        `stream` by an event at entry and joined back by an event before the down
- *        launch, so the call is ordered on `stream` like any other and can be
- *        captured into a graph (the events become edges).  Results are bit for bit
- *        those of the one-stream path.  No counterpart in the reference (XLA
- *        schedules its own streams).
+ *   decode sizes: where jtmoe_moe_forward_takes_decode_path(T, H, E, K, I, dtype) holds (bf16, at
+ *        most 64 tokens, T*K >= 2*E, 16 / 32 / 64 experts, H a multiple of 128: a decode
+ *        step), one launch runs every token through every expert's gate and up matrices --
+ *        which needs nothing of the routing -- while a few of its workgroups are the
+ *        router and write the dispatch plan; the down launch then takes the routed rows.
+ *        The workspace then holds the activations [E,T,I]; results are bit for bit those
+ *        of the other path.  That launch counts its router workgroups in one of 64 words
+ *        of device memory inside the library (zero at load, set back to zero by the
+ *        launch); the host hands the words out round-robin, so more than 64 such calls
+ *        in flight at once on one GPU are not supported.  No counterpart in the
+ *        reference (XLA decides its own fusions).
  */
-int jtmoe_moe_forward_uses_second_stream(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype);
+int jtmoe_moe_forward_takes_decode_path(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype);
 size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype);
 int jtmoe_moe_forward(const void* x, const void* w_router, const float* expert_bias,
                       const void* gate, const void* up, const void* down,

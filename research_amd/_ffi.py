@@ -60,7 +60,7 @@ PROTOTYPES: dict[str, tuple] = {
         [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr],
     ),
     "jtmoe_grouped_swiglu_gather_supported": (c_int, [c_i64, c_i64, c_i64, c_int]),
-    "jtmoe_moe_forward_uses_second_stream": (c_int, [c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),
+    "jtmoe_moe_forward_takes_decode_path": (c_int, [c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),
     "jtmoe_grouped_swiglu_gather": (
         c_int,
         [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr],

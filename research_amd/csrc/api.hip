@@ -4,7 +4,6 @@
 
 #include <cstdarg>
 #include <cstdio>
-#include <mutex>
 
 namespace jtmoe {
 
@@ -306,35 +305,6 @@ __global__ __launch_bounds__(kSmebuWaves * 64) void smebu_update_kernel(
   }
 }
 
-// A second stream per device, with the two events of a fork and join, for the one place where the
-// layer has independent work to overlap (the decode path: expert matrices streamed beside the router).
-// Default priority, created on the first use on a device and kept until the process ends.  The
-// events carry no timing; a wait takes the state of its event at the moment it is enqueued, so the
-// pair can be recorded again by the next call (the mutex covers one call's fork ... join sequence).
-struct SideStream {
-  hipStream_t stream = nullptr;
-  hipEvent_t fork = nullptr, join = nullptr;
-  bool ok = false, tried = false;
-};
-constexpr int kMaxDevices = 64;
-std::mutex g_side_mutex;
-SideStream g_side[kMaxDevices];
-
-// with g_side_mutex held
-SideStream* side_stream_locked() {
-  int device = -1;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
-  SideStream& sd = g_side[device];
-  if (!sd.tried) {
-    sd.tried = true;
-    sd.ok = hipStreamCreateWithFlags(&sd.stream, hipStreamNonBlocking) == hipSuccess &&
-            hipEventCreateWithFlags(&sd.fork, hipEventDisableTiming) == hipSuccess &&
-            hipEventCreateWithFlags(&sd.join, hipEventDisableTiming) == hipSuccess;
-    if (!sd.ok) (void)hipGetLastError();  // the caller falls back to one stream
-  }
-  return sd.ok ? &sd : nullptr;
-}
-
 struct Carve {
   unsigned char* base;
   size_t used;
@@ -455,7 +425,7 @@ extern "C" int jtmoe_smebu_update(const float* router_counts, float* momentum, f
   return check_launch("smebu_update");
 }
 
-extern "C" int jtmoe_moe_forward_uses_second_stream(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype) {
+extern "C" int jtmoe_moe_forward_takes_decode_path(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype) {
   if (T < 0 || H <= 0 || E <= 0 || K <= 0 || I <= 0 || !dtype_ok(dtype)) return 0;
   return decode_dense_supported(T, H, E, K, I, dtype) ? 1 : 0;
 }
@@ -501,52 +471,17 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
   // The router of a layer call leaves out what the dispatch behind it can do in passing: at large
   // batches the statistics (no zeroing and no finalising launch, no global atomics), at small ones
   // its finishing workgroup writes the dispatch plan as well.
-  // Decode path (a handful of tokens): the gate/up launch runs every token through every expert, which
-  // needs nothing of the routing, so the router (and the plan) run beside it on a second stream; the
-  // down launch then picks the routed rows.  The GEMM stays on the caller's stream and the router goes
-  // to the other one, not the reverse: a dependency that crosses streams costs about 10 us when the
-  // waiting stream is idle at that moment, and the router's result is there long before the GEMM ends.
-  // With a stage timer installed everything stays on the one stream, so that a stage's time is its
-  // kernels' time.
+  // Decode path (a handful of tokens): one launch runs every token through every expert's gate and up
+  // matrices, which needs nothing of the routing, and a few of its workgroups are the router and write
+  // the dispatch plan; the down launch then picks the routed rows.
   hipStream_t main_stream = as_stream(stream);
   const bool decode = !train && decode_dense_supported(T, H, E, K, I, dtype);
-  std::unique_lock<std::mutex> side_lock(g_side_mutex, std::defer_lock);  // held from the fork to the join
-  SideStream* side = nullptr;
-  if (decode && g_stage_timer == nullptr) {
-    side_lock.lock();
-    side = side_stream_locked();
-    if (side != nullptr && (hipEventRecord(side->fork, main_stream) != hipSuccess ||
-                            hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)) {
-      (void)hipGetLastError();
-      side = nullptr;
-    }
-    if (side == nullptr) side_lock.unlock();
-  }
-  const bool forked = side != nullptr;
-  hipStream_t route_stream = forked ? side->stream : main_stream;
   bool stats_done = false, plan_done = false;
-  // (forked: the expert matrices start streaming on the caller's stream before anything else is enqueued)
-  int rc = forked ? launch_gate_up_all_tokens(x, gate, up, w.act, T, H, I, E, main_stream) : JTMOE_OK;
-  if (rc == JTMOE_OK)
-    rc = router_for_layer(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
-                          expert_counts, importance, group_sizes, offsets, source_order, inverse, w.router,
-                          w.router_bytes, score_func, &stats_done, &plan_done, route_stream, forked);
-  if (rc == JTMOE_OK) {
-    stage_mark(kStageRouter, route_stream);
-    rc = dispatch_for_layer(expert_ids, weights, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes,
-                            offsets, source_order, inverse, w.packed_x, expert_counts, importance, w.dispatch,
-                            !stats_done, plan_done, route_stream);
-  }
-  if (forked) {
-    // the second stream joins again whatever happened on it (a capture of the caller's stream could not end otherwise)
-    const bool joined = hipEventRecord(side->join, side->stream) == hipSuccess &&
-                        hipStreamWaitEvent(main_stream, side->join, 0) == hipSuccess;
-    side_lock.unlock();
-    if (rc == JTMOE_OK && !joined) rc = fail(JTMOE_ELAUNCH, "moe_forward: joining the second stream failed");
-  }
-  if (rc) return rc;
+  int rc;
   if (decode) {
-    if (!forked) rc = launch_gate_up_all_tokens(x, gate, up, w.act, T, H, I, E, main_stream);
+    rc = launch_decode_gate_up_router(x, w_router, expert_bias, gate, up, w.act, T, H, E, K, I, route_scale,
+                                      score_func, expert_ids, weights, scores, expert_counts, importance, group_sizes,
+                                      offsets, source_order, inverse, w.router, main_stream);
     if (rc) return rc;
     stage_mark(kStageGateUp, main_stream);
     rc = launch_down_from_all_tokens(w.act, down, group_sizes, offsets, source_order, T, K, H, I, E, w.packed_y,
@@ -554,16 +489,29 @@ static int moe_forward_impl(const void* x, const void* w_router, const float* ex
     if (rc) return rc;
     stage_mark(kStageDown, main_stream);
     rc = check_launch("grouped gemm");
-  } else if (train)
-    rc = jtmoe_grouped_swiglu_train(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
-                                    gate_pre, up_pre, w.act, w.packed_y, stream);
-  else if (gather)
-    rc = jtmoe_grouped_swiglu_gather(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
-                                     w.act, w.packed_y, stream);
-  else
-    rc = jtmoe_grouped_swiglu(w.packed_x, gate, up, down, group_sizes, offsets, T * K, H, I, E, dtype, w.act,
-                              w.packed_y, stream);
+  } else {
+    rc = router_for_layer(x, w_router, expert_bias, T, H, E, K, route_scale, dtype, expert_ids, weights, scores,
+                          expert_counts, importance, group_sizes, offsets, source_order, inverse, w.router,
+                          w.router_bytes, score_func, &stats_done, &plan_done, main_stream);
+    if (rc) return rc;
+    stage_mark(kStageRouter, main_stream);
+    rc = dispatch_for_layer(expert_ids, weights, (T > 0 && !gather) ? x : nullptr, T, H, E, K, dtype, group_sizes,
+                            offsets, source_order, inverse, w.packed_x, expert_counts, importance, w.dispatch,
+                            !stats_done, plan_done, main_stream);
+  }
   if (rc) return rc;
+  if (!decode) {  // (the decode path has enqueued both of its GEMM launches above)
+    if (train)
+      rc = jtmoe_grouped_swiglu_train(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
+                                      gate_pre, up_pre, w.act, w.packed_y, stream);
+    else if (gather)
+      rc = jtmoe_grouped_swiglu_gather(x, source_order, gate, up, down, group_sizes, offsets, T, K, H, I, E, dtype,
+                                       w.act, w.packed_y, stream);
+    else
+      rc = jtmoe_grouped_swiglu(w.packed_x, gate, up, down, group_sizes, offsets, T * K, H, I, E, dtype, w.act,
+                                w.packed_y, stream);
+    if (rc) return rc;
+  }
   if (Is > 0) {
     if (train)
       rc = jtmoe_shared_swiglu_train(x, shared_gate, shared_up, shared_down, T, H, Is, dtype, shared_gate_pre,

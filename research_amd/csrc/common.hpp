@@ -128,23 +128,28 @@ int dispatch_for_layer(const int32_t* expert_ids, const void* weights, const voi
 // path gets them from its one finishing workgroup); if not, the caller's dispatch computes them from
 // the ids and weights.  *plan_done says whether group_sizes / offsets / source_order / inverse have
 // been written as well (the finishing workgroup of the small-batch router goes on to the plan while
-// it still holds the ids in LDS).  beside_gemm: another launch is filling the CUs while this one runs.
+// it still holds the ids in LDS).
 int router_for_layer(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H, int64_t E,
                      int64_t K, double route_scale, int dtype, int32_t* expert_ids, void* weights, float* scores,
                      float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
                      int32_t* source_order, int32_t* inverse, void* workspace, size_t workspace_bytes,
-                     int score_func, bool* stats_done, bool* plan_done, hipStream_t stream, bool beside_gemm = false);
+                     int score_func, bool* stats_done, bool* plan_done, hipStream_t stream);
 
 
-// grouped_gemm.hip: the decode path of the layer (a handful of tokens, nearly every expert chosen by some
-// token).  The gate/up launch runs ALL T tokens through every expert -- act_full [E][T][I] -- which
-// needs nothing of the routing, so it can run beside the router; the down launch then takes packed
-// row j from act_full[expert of j][source_order[j] / K].  A tile is 64 rows tall whether it holds an
-// expert's few routed rows or all T <= 64 tokens, so the launches stream the same expert matrices in
-// the same time, and the rows that were routed come out bit for bit as from the gathering launch.
+// The decode path of the layer (a handful of tokens, nearly every expert chosen by some token).  A tile is
+// 64 rows tall whether it holds an expert's few routed rows or all T <= 64 tokens, so ONE launch runs every
+// token through every expert's gate and up matrices -- act_full [E][T][I], which needs nothing of the
+// routing -- while a few of its workgroups are the router and write the dispatch plan (router.hip); the
+// down launch (grouped_gemm.hip) then takes packed row j from act_full[expert of j][source_order[j] / K].
+// The launches stream the same expert matrices in the same time as the gathering ones, the router's
+// dependent steps no longer stand in front of them, and the rows that were routed come out bit for bit as
+// from the gathering launch.
 bool decode_dense_supported(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype);
-int launch_gate_up_all_tokens(const void* x, const void* gate, const void* up, void* act_full, int64_t T, int64_t H,
-                              int64_t I, int64_t E, hipStream_t stream);
+int launch_decode_gate_up_router(const void* x, const void* w_router, const float* expert_bias, const void* gate,
+                                 const void* up, void* act_full, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I,
+                                 double route_scale, int score_func, int32_t* expert_ids, void* weights, float* scores,
+                                 float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
+                                 int32_t* source_order, int32_t* inverse, void* router_workspace, hipStream_t stream);
 int launch_down_from_all_tokens(const void* act_full, const void* down, const int32_t* group_sizes,
                                 const int32_t* offsets, const int32_t* source_order, int64_t T, int64_t K, int64_t H,
                                 int64_t I, int64_t E, void* packed_y, hipStream_t stream);

@@ -116,11 +116,13 @@ struct TileCoord {
 // Workgroup id -> (m-tile, n-tile).  Consecutive workgroup ids go round-robin to the 8 XCDs, so
 // each XCD gets a contiguous range of the logical order, and that order is walked in groups of
 // group_m m-tiles x all n-tiles so that neighbours share operand panels in their L2.
-__device__ __forceinline__ TileCoord xcd_tile_order(int mtiles, int ntiles_n, int group_m) {
+// (block / blocks: this workgroup's index among the workgroups that share out the tiles, and their number --
+// the launch's own unless other workgroups of the launch do something else)
+__device__ __forceinline__ TileCoord xcd_tile_order(int mtiles, int ntiles_n, int group_m, int block, int blocks) {
   TileCoord t;
   const int total = mtiles * ntiles_n;
-  const int per_xcd = (int)gridDim.x >> 3;
-  const int logical = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  const int per_xcd = blocks >> 3;
+  const int logical = (block & 7) * per_xcd + (block >> 3);
   if (logical >= total) {
     t.mt = -1;
     t.nt = 0;
@@ -139,14 +141,14 @@ __device__ __forceinline__ TileCoord xcd_tile_order(int mtiles, int ntiles_n, in
 // and only `mtiles` of them exist (group sizes live on the device): the XCD ranges are cut from the
 // real count, so that the surplus workgroups are spread over all XCDs instead of idling one of them.
 // Requires gridDim.x / 8 >= ceil(mtiles * ntiles_n / 8), which the bound guarantees.
-__device__ __forceinline__ TileCoord xcd_tile_order_balanced(int mtiles, int ntiles_n, int group_m) {
+__device__ __forceinline__ TileCoord xcd_tile_order_balanced(int mtiles, int ntiles_n, int group_m, int block) {
   TileCoord t;
   t.mt = -1;
   t.nt = 0;
   const int total = mtiles * ntiles_n;
   const int per_xcd = (total + 7) >> 3;
-  const int idx = (int)blockIdx.x >> 3;
-  const int logical = ((int)blockIdx.x & 7) * per_xcd + idx;
+  const int idx = block >> 3;
+  const int logical = (block & 7) * per_xcd + idx;
   if (idx >= per_xcd || logical >= total) return t;
   const int group_span = group_m * ntiles_n;
   const int group = logical / group_span;
@@ -155,6 +157,13 @@ __device__ __forceinline__ TileCoord xcd_tile_order_balanced(int mtiles, int nti
   t.nt = in_group / gm;
   t.mt = group * group_m + (in_group - t.nt * gm);
   return t;
+}
+
+__device__ __forceinline__ TileCoord xcd_tile_order(int mtiles, int ntiles_n, int group_m) {
+  return xcd_tile_order(mtiles, ntiles_n, group_m, (int)blockIdx.x, (int)gridDim.x);
+}
+__device__ __forceinline__ TileCoord xcd_tile_order_balanced(int mtiles, int ntiles_n, int group_m) {
+  return xcd_tile_order_balanced(mtiles, ntiles_n, group_m, (int)blockIdx.x);
 }
 
 // Second half of every epilogue: a wave has parked its WM x WNO block of bf16 results in its own

@@ -304,24 +304,7 @@ int validate_gemm(const char* what, int64_t rows, int64_t H, int64_t I, int64_t 
 
 }  // namespace
 
-// ---- the decode path of the layer (declared in common.hpp) ----
-constexpr int64_t kDecodeMaxTokens = 64;  // one 64-row tile per expert holds every token
-
-bool decode_dense_supported(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype) {
-  // all tokens through every expert pays when nearly every expert would be streamed anyway: with
-  // T * K >= 2 E assignments thrown at E experts fewer than e^-2 = 14 % of them stay without a row
-  return dtype == JTMOE_BF16 && T > 0 && T <= kDecodeMaxTokens && T * K >= 2 * E && tiny_groups(T * K, E) &&
-         E <= JTMOE_MAX_EXPERTS && H % 64 == 0 && I % 64 == 0 && H * I < ((int64_t)1 << 30) &&
-         E * T * (I > H ? I : H) < ((int64_t)1 << 30);
-}
-
-int launch_gate_up_all_tokens(const void* x, const void* gate, const void* up, void* act_full, int64_t T, int64_t H,
-                              int64_t I, int64_t E, hipStream_t stream) {
-  if (!fast_ok(x, gate, up, act_full, H, I)) return fail(JTMOE_EINVAL, "moe_forward: operands must be 16-byte aligned");
-  return launch_fast<GateUpTinyCfg>(x, gate, up, act_full, nullptr, nullptr, E * T, H, I, E, stream, nullptr, 1, 0,
-                                    nullptr, nullptr, /*uniform_rows=*/T);
-}
-
+// ---- the down launch of the layer's decode path (declared in common.hpp) ----
 int launch_down_from_all_tokens(const void* act_full, const void* down, const int32_t* group_sizes,
                                 const int32_t* offsets, const int32_t* source_order, int64_t T, int64_t K, int64_t H,
                                 int64_t I, int64_t E, void* packed_y, hipStream_t stream) {

@@ -232,13 +232,16 @@ __device__ __forceinline__ void store_transposed_accumulators(const f32x16_t (&a
   }
 }
 
+// One tile per workgroup.  block / blocks: this workgroup's index among the workgroups that share out the
+// tiles and their number (the launch's own in grouped_gemm_dma_kernel below; a launch may also give some of
+// its workgroups other work, see the decode launch of the router).
 template <typename Cfg>
-__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::MIN_WAVES_PER_EU))) void grouped_gemm_dma_kernel(
+__device__ __forceinline__ void grouped_gemm_dma_tile(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
     uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
     int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
-    int a_rows, uint16_t* __restrict__ save0 = nullptr, uint16_t* __restrict__ save1 = nullptr, int uniform_rows = 0,
-    int a_group_rows = 0) {
+    int a_rows, uint16_t* __restrict__ save0, uint16_t* __restrict__ save1, int uniform_rows, int a_group_rows,
+    int block, int blocks) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, NSTAGE = Cfg::NSTAGE;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, WM = Cfg::WM, WN = Cfg::WN;
   constexpr int CPRA = Cfg::CPRA;
@@ -253,7 +256,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::MI
     // Every group takes the SAME uniform_rows rows of A (all tokens through every expert: the decode
     // path, which does not wait for the routing): group e writes rows [e, e + 1) * uniform_rows of C.
     const int per_group = (uniform_rows + BM - 1) / BM;
-    tc = xcd_tile_order(E * per_group, ntiles_n, Cfg::GROUP_M);
+    tc = xcd_tile_order(E * per_group, ntiles_n, Cfg::GROUP_M, block, blocks);
     if (tc.mt < 0) return;
     tr.expert = tc.mt / per_group;
     const int local_row0 = (tc.mt - tr.expert * per_group) * BM;
@@ -262,11 +265,11 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::MI
     a_row0 = local_row0;
   } else if (group_sizes) {
     const GroupScan scan = group_scan(BM, group_sizes, E);
-    tc = xcd_tile_order_balanced(scan.total, ntiles_n, Cfg::GROUP_M);
+    tc = xcd_tile_order_balanced(scan.total, ntiles_n, Cfg::GROUP_M, block);
     if (tc.mt < 0) return;
     tr = locate_tile(scan, tc.mt, BM, offsets);
   } else {
-    tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M);
+    tc = xcd_tile_order(mtiles, ntiles_n, Cfg::GROUP_M, block, blocks);
     if (tc.mt < 0) return;
     tr = find_tile_wave(tc.mt, BM, nullptr, nullptr, E, dense_rows);
   }
@@ -491,6 +494,18 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::MI
     else
       store_wave_block<WM, WNO, CS, true>(cw, lane, out, N, (size_t)tr.row0 + row_base, tr.rows - row_base, col0);
   }
+}
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::MIN_WAVES_PER_EU))) void grouped_gemm_dma_kernel(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
+    uint16_t* __restrict__ C, const int32_t* __restrict__ group_sizes, const int32_t* __restrict__ offsets, int E,
+    int dense_rows, int Kdim, int N, int mtiles, int ntiles_n, const int32_t* __restrict__ row_map, int row_div,
+    int a_rows, uint16_t* __restrict__ save0 = nullptr, uint16_t* __restrict__ save1 = nullptr, int uniform_rows = 0,
+    int a_group_rows = 0) {
+  grouped_gemm_dma_tile<Cfg>(A, B0, B1, C, group_sizes, offsets, E, dense_rows, Kdim, N, mtiles, ntiles_n, row_map,
+                             row_div, a_rows, save0, save1, uniform_rows, a_group_rows, (int)blockIdx.x,
+                             (int)gridDim.x);
 }
 
 // ---------------------------------------------------------------------------------------------

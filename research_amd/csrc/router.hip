@@ -12,6 +12,9 @@
 // logits and can be reproduced bit for bit on a CPU.
 #include "common.hpp"
 #include "dispatch_small.hpp"
+#include "grouped_gemm_dma.hpp"
+
+#include <atomic>
 
 #include <mutex>
 
@@ -411,12 +414,7 @@ __global__ __launch_bounds__(256) void router_kernel(
 // is stored and read with the transposing ds_read_b64_tr_b16.
 // Requires H % 64 == 0 and E in {16, 32, 64, 128, 256}.
 // ---------------------------------------------------------------------------
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(8))) short s16x8_t;
-typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
-constexpr int kBufferFlags = 0x00020000;
 constexpr int kRouterKC = 64;  // k rows of the router matrix per LDS stage
 constexpr int kSplitKC = 128;  // k rows per LDS stage of the small-batch kernels; the unit the slices are cut in
 constexpr int kPartialMaxSlices = 8;
@@ -592,12 +590,14 @@ __host__ __device__ inline size_t router_split_smem_bytes(int E, int K) {
 // kPartial: the grid's y dimension shares out the slices; a workgroup then only writes the unrounded
 // sum of its slice, partial_out[slice][token][expert], and router_finish_kernel adds the slices in
 // order and does the rest.  Otherwise the workgroup walks all slices itself.
+// (token_block / slice: the workgroup's place in the launch's grid -- blockIdx.x / blockIdx.y in
+// router_mfma_split_kernel; the decode launch hands them out among its own workgroups)
 template <int NB, bool kPartial>
-__global__ __launch_bounds__(256) void router_mfma_split_kernel(
+__device__ __forceinline__ void router_split_body(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
     int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
     float* __restrict__ scores, float* __restrict__ logits_out, void* ws, float* __restrict__ partial_out,
-    int score_func) {
+    int score_func, int token_block, int slice) {
   constexpr int kThreads = 256, kTokens = 16;
   constexpr int E = NB * 16;
   constexpr int WS = E + 32;
@@ -611,7 +611,7 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool has_cols = wave < NB;  // with fewer than four column blocks some waves only help to stage the matrix
-  const int t0 = blockIdx.x * kTokens;
+  const int t0 = token_block * kTokens;
   const int nrows = min(kTokens, tokens - t0);
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(x + (size_t)t0 * H), 0, nrows * H * 2, kBufferFlags);
@@ -654,7 +654,7 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
   const int w_lane = ((lane >> 4) * 8 + ((lane & 15) >> 2)) * WS + 4 * (lane & 3);
   // this workgroup's chunks: one slice of them, or all
   const int slice_chunks = router_slice_rows(H) / kSplitKC;
-  const int chunk0 = kPartial ? (int)blockIdx.y * slice_chunks : 0;
+  const int chunk0 = kPartial ? slice * slice_chunks : 0;
   const int nchunks = kPartial ? min(slice_chunks, H / kSplitKC - chunk0) : H / kSplitKC;
   const int kbase = chunk0 * kSplitKC;
   int in_slice = 0;
@@ -716,7 +716,7 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
         for (int i = 0; i < 4; ++i) {
           const int t = 4 * (lane >> 4) + i;
           if (t < nrows && wave + 4 * b < NB)
-            partial_out[((size_t)blockIdx.y * tokens + t0 + t) * E + (wave + 4 * b) * 16 + (lane & 15)] = acc[b][i];
+            partial_out[((size_t)slice * tokens + t0 + t) * E + (wave + 4 * b) * 16 + (lane & 15)] = acc[b][i];
         }
     }
     return;
@@ -738,6 +738,16 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
                                                logits_out, router_scratch(ws, E), score_func);
 }
 
+template <int NB, bool kPartial>
+__global__ __launch_bounds__(256) void router_mfma_split_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const float* __restrict__ bias, int tokens,
+    int H, int K, float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights,
+    float* __restrict__ scores, float* __restrict__ logits_out, void* ws, float* __restrict__ partial_out,
+    int score_func) {
+  router_split_body<NB, kPartial>(x, w, bias, tokens, H, K, route_scale, ids, weights, scores, logits_out, ws,
+                                  partial_out, score_func, (int)blockIdx.x, (int)blockIdx.y);
+}
+
 // Second half of the small-batch router: one workgroup adds the slices of partial sums in slice
 // order, rounds to bf16 (the projection's output dtype) and runs the epilogue for every token of
 // the call, so the statistics need neither the zeroing nor the finalising launch.
@@ -747,7 +757,7 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(
 // the place of the score tile, which is dead by then.  Requires tokens * K <= kSmallMaxAssignments
 // and E <= 4 * kTok.
 template <int kTok, bool kPlan>
-__global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
+__device__ __forceinline__ void router_finish_body(
     const float* __restrict__ partial, int slices, const float* __restrict__ bias, int tokens, int E, int K,
     float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights, float* __restrict__ scores,
     float* __restrict__ logits_out, float* __restrict__ counts, float* __restrict__ importance,
@@ -780,6 +790,76 @@ __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
   }
 }
 
+template <int kTok, bool kPlan>
+__global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
+    const float* __restrict__ partial, int slices, const float* __restrict__ bias, int tokens, int E, int K,
+    float route_scale, int32_t* __restrict__ ids, bf16_raw* __restrict__ weights, float* __restrict__ scores,
+    float* __restrict__ logits_out, float* __restrict__ counts, float* __restrict__ importance,
+    int32_t* __restrict__ group_sizes, int32_t* __restrict__ offsets, int32_t* __restrict__ source_order,
+    int32_t* __restrict__ inverse, int score_func) {
+  router_finish_body<kTok, kPlan>(partial, slices, bias, tokens, E, K, route_scale, ids, weights, scores, logits_out,
+                                  counts, importance, group_sizes, offsets, source_order, inverse, score_func);
+}
+
+// ---------------------------------------------------------------------------
+// The decode launch: ONE launch in which most workgroups stream the gate and up matrices (every token
+// through every expert, grouped_gemm_dma_tile in its uniform mode -- nothing of that needs the routing)
+// and the first token_blocks * slices workgroups are the small-batch router: each computes the partial
+// sums of its (token block, slice), counts itself in, and the last of them to arrive adds the slices up
+// in slice order and runs the epilogue and the dispatch plan (router_finish_body) -- the same arithmetic
+// in the same order as the two-launch form, so the same bits.  The router's 21 us of dependent steps
+// then run beside the 115 us of weight streaming instead of in front of it, with no second stream and
+// no dependency between launches other than the stream's own order.
+// The arrival counter of a launch is one of kDecodeSlots words of device memory that are zero when the
+// library is loaded; the last workgroup to arrive sets its word back to zero.  The host hands the slots
+// out round-robin, so launches that overlap on one GPU (from several streams) use different words unless
+// more than kDecodeSlots of them are in flight at once.
+// ---------------------------------------------------------------------------
+constexpr int kDecodeSlots = 64;
+__device__ unsigned g_decode_arrivals[kDecodeSlots];
+std::atomic<unsigned> g_decode_next_slot{0};
+
+template <int NB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void decode_gate_up_router_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up,
+    uint16_t* __restrict__ act_full, int T, int H, int I, int mtiles, int ntiles_n,
+    const uint16_t* __restrict__ w_router, const float* __restrict__ bias, int K, float route_scale, int score_func,
+    int32_t* __restrict__ ids, bf16_raw* __restrict__ weights, float* __restrict__ scores,
+    float* __restrict__ counts, float* __restrict__ importance, int32_t* __restrict__ group_sizes,
+    int32_t* __restrict__ offsets, int32_t* __restrict__ source_order, int32_t* __restrict__ inverse,
+    float* __restrict__ partial, int token_blocks, int slices, int slot) {
+  constexpr int E = NB * 16;
+  const int router_blocks = token_blocks * slices;
+  if ((int)blockIdx.x >= router_blocks) {
+    grouped_gemm_dma_tile<GateUpTinyCfg>(x, gate, up, act_full, nullptr, nullptr, E, E * T, H, I, mtiles, ntiles_n,
+                                         nullptr, 1, 0, nullptr, nullptr, /*uniform_rows=*/T, 0,
+                                         (int)blockIdx.x - router_blocks, (int)gridDim.x - router_blocks);
+    return;
+  }
+  __shared__ int is_last;
+  const int token_block = (int)blockIdx.x % token_blocks, slice = (int)blockIdx.x / token_blocks;
+  router_split_body<NB, true>(x, w_router, bias, T, H, K, route_scale, ids, weights, scores, nullptr, nullptr, partial,
+                              score_func, token_block, slice);
+  // Hand-over.  Every thread waits until its own stores have reached the L2 (on this part stores count in
+  // vmcnt); after the barrier one thread releases them to the device (the fence writes the L2's dirty
+  // lines back, so that the other XCDs can see them) and counts the workgroup in.  The workgroup that
+  // finds everyone else counted acquires with one fence (it invalidates this CU's L1 and the stale lines
+  // of its L2) before any of its threads reads the others' sums.  One fence per workgroup, not one per
+  // thread: each is an operation on whole caches.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    is_last = atomicAdd(&g_decode_arrivals[slot], 1u) == (unsigned)(router_blocks - 1);
+    if (is_last) __threadfence();
+  }
+  __syncthreads();
+  if (!is_last) return;
+  router_finish_body<64, true>(partial, slices, bias, T, E, K, route_scale, ids, weights, scores, nullptr, counts,
+                               importance, group_sizes, offsets, source_order, inverse, score_func);
+  if (threadIdx.x == 0) g_decode_arrivals[slot] = 0u;
+}
+
 template <typename KernelT>
 int set_max_smem(KernelT kernel, size_t bytes) {
   if (bytes <= 64 * 1024) return JTMOE_OK;
@@ -798,11 +878,6 @@ struct LayerPlan {
   int32_t* inverse;
   bool stats_done;
   bool plan_done;
-  // the call runs beside a launch that fills the CUs (the decode path's gate/up): the finishing
-  // workgroup then takes its 64-token form where that holds the batch -- 256 threads and a fifth of
-  // the LDS, which a CU can place next to three resident GEMM workgroups; the 1024-thread form would
-  // wait for a CU to drain
-  bool beside_gemm;
 };
 
 template <typename T, bool kFromLogits>
@@ -828,9 +903,7 @@ int launch_router(const void* x, const void* w, const float* logits_in, const fl
         return fail(JTMOE_EUNSUPPORTED, "router: E=%lld K=%lld needs %zu bytes of LDS", (long long)E, (long long)K, smem);
       // Two launches when one workgroup can hold the epilogue of the whole call: partial sums over
       // k slices from many workgroups, then the finishing workgroup.
-      const int finish_tok = (layer != nullptr && layer->beside_gemm && tokens <= 64)                  ? 64
-                             : router_smem_bytes((int)E, (int)K, 256) <= 160 * 1024 ? 256
-                                                                                    : 64;
+      const int finish_tok = router_smem_bytes((int)E, (int)K, 256) <= 160 * 1024 ? 256 : 64;
       if (tokens > 0 && tokens <= finish_tok && router_smem_bytes((int)E, (int)K, finish_tok) <= 160 * 1024) {
         const int slice_rows = router_slice_rows((int)H);
         const int slices = (int)((H + slice_rows - 1) / slice_rows);
@@ -966,11 +1039,66 @@ int validate_router(int64_t T, int64_t H, int64_t E, int64_t K, double route_sca
 
 }  // namespace
 
+// ---- the decode path of the layer (declared in common.hpp) ----
+bool decode_dense_supported(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype) {
+  // Every token through every expert pays when nearly every expert would be streamed anyway: with
+  // T * K >= 2 E assignments thrown at E experts fewer than e^-2 = 14 % of them stay without a row.  One
+  // 64-row tile per expert holds every token; the router's workgroups inside the launch need the matrix-core
+  // projection (H a multiple of 128) and, so that three workgroups still fit a CU beside each other, a
+  // router matrix stage of at most 53 KB (E <= 64); the plan needs E <= 256 and T * K <= kSmallMaxAssignments.
+  return dtype == JTMOE_BF16 && T > 0 && T <= 64 && T * K >= 2 * E && T * K <= 32 * E &&
+         (E == 16 || E == 32 || E == 64) && K <= JTMOE_MAX_TOP_K && K <= E && H % kSplitKC == 0 && I % 64 == 0 &&
+         H * I < ((int64_t)1 << 30) && E * T * (I > H ? I : H) < ((int64_t)1 << 30) &&
+         T * K <= kSmallMaxAssignments;
+}
+
+int launch_decode_gate_up_router(const void* x, const void* w_router, const float* expert_bias, const void* gate,
+                                 const void* up, void* act_full, int64_t T, int64_t H, int64_t E, int64_t K, int64_t I,
+                                 double route_scale, int score_func, int32_t* expert_ids, void* weights, float* scores,
+                                 float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
+                                 int32_t* source_order, int32_t* inverse, void* router_workspace, hipStream_t stream) {
+  if (!(aligned16(x) && aligned16(w_router) && aligned16(gate) && aligned16(up) && aligned16(act_full)))
+    return fail(JTMOE_EINVAL, "moe_forward: operands must be 16-byte aligned");
+  const int token_blocks = (int)((T + 15) / 16);
+  const int slice_rows = router_slice_rows((int)H);
+  const int slices = (int)((H + slice_rows - 1) / slice_rows);
+  float* partial = reinterpret_cast<float*>(static_cast<unsigned char*>(router_workspace) + router_scratch_bytes(E));
+  size_t smem = GateUpTinyCfg::SMEM_BYTES;
+  if (router_split_smem_bytes((int)E, (int)K) > smem) smem = router_split_smem_bytes((int)E, (int)K);
+  if (router_smem_bytes((int)E, (int)K, 64) > smem) smem = router_smem_bytes((int)E, (int)K, 64);
+  if (smem > 53 * 1024) return fail(JTMOE_EUNSUPPORTED, "moe_forward: decode launch needs %zu bytes of LDS", smem);
+  const int64_t mtiles = E * ((T + GateUpTinyCfg::BM - 1) / GateUpTinyCfg::BM);
+  const int64_t nt = (I + GateUpTinyCfg::BN - 1) / GateUpTinyCfg::BN;
+  const int64_t grid = (int64_t)token_blocks * slices + gemm_grid(mtiles, nt);
+  const int slot = (int)(g_decode_next_slot.fetch_add(1u, std::memory_order_relaxed) % kDecodeSlots);
+#define JT_DECODE_CASE(NB)                                                                                       \
+  case NB * 16: {                                                                                                \
+    auto kernel = decode_gate_up_router_kernel<NB>;                                                              \
+    int rc = set_max_smem(kernel, smem);                                                                         \
+    if (rc) return rc;                                                                                           \
+    kernel<<<(unsigned)grid, 256, smem, stream>>>(                                                               \
+        static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up),   \
+        static_cast<uint16_t*>(act_full), (int)T, (int)H, (int)I, (int)mtiles, (int)nt,                          \
+        static_cast<const uint16_t*>(w_router), expert_bias, (int)K, (float)route_scale, score_func, expert_ids, \
+        static_cast<bf16_raw*>(weights), scores, expert_counts, importance, group_sizes, offsets, source_order,  \
+        inverse, partial, token_blocks, slices, slot);                                                           \
+  } break;
+  switch ((int)E) {
+    JT_DECODE_CASE(1)
+    JT_DECODE_CASE(2)
+    JT_DECODE_CASE(4)
+    default:
+      return fail(JTMOE_EUNSUPPORTED, "moe_forward: decode launch for E=%lld", (long long)E);
+  }
+#undef JT_DECODE_CASE
+  return check_launch("decode gate/up + router");
+}
+
 int router_for_layer(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H, int64_t E,
                      int64_t K, double route_scale, int dtype, int32_t* expert_ids, void* weights, float* scores,
                      float* expert_counts, float* importance, int32_t* group_sizes, int32_t* offsets,
                      int32_t* source_order, int32_t* inverse, void* workspace, size_t workspace_bytes,
-                     int score_func, bool* stats_done, bool* plan_done, hipStream_t s, bool beside_gemm) {
+                     int score_func, bool* stats_done, bool* plan_done, hipStream_t s) {
   int rc = validate_router(T, H, E, K, route_scale, dtype, true);
   if (rc) return rc;
   JT_REQUIRE(score_func_ok(score_func), "router: unknown score function %d", score_func);
@@ -979,7 +1107,7 @@ int router_for_layer(const void* x, const void* w_router, const float* expert_bi
   JT_REQUIRE(group_sizes && offsets && (T == 0 || (source_order && inverse)), "router: null pointer argument");
   if (workspace_bytes < jtmoe_router_workspace_bytes(E))
     return fail(JTMOE_EWORKSPACE, "router: workspace %zu < %zu bytes", workspace_bytes, jtmoe_router_workspace_bytes(E));
-  LayerPlan layer{group_sizes, offsets, source_order, inverse, false, false, beside_gemm};
+  LayerPlan layer{group_sizes, offsets, source_order, inverse, false, false};
   if (dtype == JTMOE_BF16)
     rc = launch_router<bf16_raw, false>(x, w_router, nullptr, expert_bias, T, H, E, K, route_scale, expert_ids, weights,
                                         scores, expert_counts, importance, nullptr, workspace, s, score_func, &layer);

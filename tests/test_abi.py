@@ -56,12 +56,12 @@ def test_workspace_sizing_is_pure_host_arithmetic():
     assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, 7) == 0  # unknown dtype
     # the decode path (second stream, activations of all tokens through every expert) and its workspace
     bf = _ffi.JTMOE_BF16
-    assert lib.jtmoe_moe_forward_uses_second_stream(64, H, E, K, I, bf) == 1
-    assert lib.jtmoe_moe_forward_uses_second_stream(16, H, E, K, I, bf) == 1   # T * K = 2 * E
-    assert lib.jtmoe_moe_forward_uses_second_stream(15, H, E, K, I, bf) == 0
-    assert lib.jtmoe_moe_forward_uses_second_stream(65, H, E, K, I, bf) == 0
-    assert lib.jtmoe_moe_forward_uses_second_stream(T, H, E, K, I, bf) == 0
-    assert lib.jtmoe_moe_forward_uses_second_stream(64, H, E, K, I, _ffi.JTMOE_F32) == 0
+    assert lib.jtmoe_moe_forward_takes_decode_path(64, H, E, K, I, bf) == 1
+    assert lib.jtmoe_moe_forward_takes_decode_path(16, H, E, K, I, bf) == 1   # T * K = 2 * E
+    assert lib.jtmoe_moe_forward_takes_decode_path(15, H, E, K, I, bf) == 0
+    assert lib.jtmoe_moe_forward_takes_decode_path(65, H, E, K, I, bf) == 0
+    assert lib.jtmoe_moe_forward_takes_decode_path(T, H, E, K, I, bf) == 0
+    assert lib.jtmoe_moe_forward_takes_decode_path(64, H, E, K, I, _ffi.JTMOE_F32) == 0
     assert lib.jtmoe_workspace_bytes(64, H, E, K, I, 0, bf) >= 2 * (E * 64 * I + 64 * K * H)
     assert lib.jtmoe_router_workspace_bytes(E) >= 12 * E
     assert lib.jtmoe_dispatch_workspace_bytes(A, E) >= 4 * E * ((A + 1023) // 1024)

@@ -123,23 +123,27 @@ def check_random_layer_shapes(gpu, seed: int, cases: int) -> None:
         assert bool(torch.isfinite(layer.y.float()).all()), tag
 
 
-# (tokens, hidden, experts, top_k, d_ff, shared width): at most 64 tokens, tokens * top_k >= 2 * experts
+# (tokens, hidden, experts, top_k, d_ff, shared width): at most 64 tokens, tokens * top_k >= 2 * experts,
+# 16 / 32 / 64 experts, hidden a multiple of 128
 DECODE_CASES = [
     (64, 2048, 64, 8, 1408, 0),   # the decode shape of the benchmark
     (64, 2048, 64, 8, 128, 256),  # with shared experts
     (16, 256, 64, 8, 64, 0),      # tokens * top_k = 2 * experts: the smallest batch that takes the path
-    (40, 128, 16, 2, 192, 0),
-    (33, 192, 8, 8, 64, 64),      # every token picks every expert
+    (40, 128, 16, 2, 192, 0),     # one slice of the hidden dimension, three token blocks (the last ragged)
+    (64, 256, 32, 4, 128, 0),
+    (48, 384, 16, 2, 64, 64),     # three slices
+    (1, 1920, 16, 16, 64, 0),     # one token that picks every expert; 15 chunks: slices of two, the last of one
+    (33, 192, 8, 8, 64, 64),      # 8 experts, hidden not a multiple of 128: the ordinary path
     (15, 256, 64, 8, 64, 0),      # one token short: the ordinary path (the comparison must hold either way)
 ]
 
 
 @pytest.mark.parametrize("tokens,hidden,experts,top_k,d_ff,shared_width", DECODE_CASES)
 def test_decode_path_equals_the_stand_alone_operators(gpu, tokens, hidden, experts, top_k, d_ff, shared_width):
-    """At decode-sized batches the layer runs every token through every expert beside the router (on a
-    second stream) and the down projection picks the routed rows.  The output must equal, bit for bit,
-    router -> dispatch -> gathering grouped SwiGLU -> combine called one by one, twice in a row, and
-    through a workspace that a larger call has used in between."""
+    """At decode-sized batches one launch runs every token through every expert while a few of its
+    workgroups are the router and write the dispatch plan, and the down projection picks the routed rows.
+    Every output must equal, bit for bit, router -> dispatch -> gathering grouped SwiGLU -> combine called
+    one by one, twice in a row, and through a workspace that a larger call has used in between."""
     rng = np.random.default_rng(tokens * 131 + experts)
     x = dev(rng.standard_normal((tokens, hidden)).astype(np.float32), gpu, "bf16")
     w_router = dev((rng.standard_normal((hidden, experts)) * 0.1).astype(np.float32), gpu, "bf16")
@@ -158,7 +162,10 @@ def test_decode_path_equals_the_stand_alone_operators(gpu, tokens, hidden, exper
 
     first = ops.moe_forward(x, w_router, None, gate, up, down, top_k, 1.0, shared=shared)
     assert torch.equal(first.y, want)
-    assert torch.equal(first.source_order, plan.source_order) and torch.equal(first.expert_ids, route.expert_ids)
+    for name in ("expert_ids", "weights", "scores", "expert_counts", "importance"):
+        assert torch.equal(getattr(first, name), getattr(route, name)), name
+    for name in ("group_sizes", "offsets", "source_order", "inverse"):
+        assert torch.equal(getattr(first, name), getattr(plan, name)), name
     big = dev(rng.standard_normal((300, hidden)).astype(np.float32), gpu, "bf16")
     ops.moe_forward(big, w_router, None, gate, up, down, top_k, 1.0, shared=shared)  # other rows through the same workspace
     again = ops.moe_forward(x, w_router, None, gate, up, down, top_k, 1.0, shared=shared)
@@ -167,8 +174,8 @@ def test_decode_path_equals_the_stand_alone_operators(gpu, tokens, hidden, exper
 
 
 def test_decode_path_follows_work_on_the_callers_stream(gpu):
-    """The second stream starts only when the caller's stream has reached the call (its input may still
-    be being written there) and the caller's stream continues only when the second stream is done."""
+    """The call is ordered on the caller's stream like any other: its input may still be being written
+    there when the call is enqueued, and its output is read there right after."""
     rng = np.random.default_rng(77)
     T, H, E, K, I = 64, 512, 64, 8, 128
     w_router = dev((rng.standard_normal((H, E)) * 0.1).astype(np.float32), gpu, "bf16")
