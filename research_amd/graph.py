@@ -7,9 +7,7 @@ once and replay the same kernels with a single launch.  The reference gets the e
 ``jax.jit`` (its decode step, blocks.py:262-290, runs inside one compiled program).
 
 The library's forward path only enqueues kernels (no allocation, no memset, no synchronisation),
-so it can be captured as it is -- also at decode sizes, where the call forks part of its work onto a
-second stream and joins it again with events: the second stream joins the capture and the events
-become edges of the graph.  Shapes are fixed at capture; the caller copies new inputs into
+so it can be captured as it is.  Shapes are fixed at capture; the caller copies new inputs into
 ``x`` (and may update the parameters in place) and calls ``replay()``.
 """
 

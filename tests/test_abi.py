@@ -54,7 +54,7 @@ def test_workspace_sizing_is_pure_host_arithmetic():
     assert odd >= 2 * (A * (H + 8) + A * I + A * (H + 8) + T * Is + T * (H + 8))
     assert lib.jtmoe_workspace_bytes(0, H, E, K, I, 0, _ffi.JTMOE_BF16) > 0
     assert lib.jtmoe_workspace_bytes(T, H, E, K, I, Is, 7) == 0  # unknown dtype
-    # the decode path (second stream, activations of all tokens through every expert) and its workspace
+    # the decode path (activations of all tokens through every expert) and its workspace
     bf = _ffi.JTMOE_BF16
     assert lib.jtmoe_moe_forward_takes_decode_path(64, H, E, K, I, bf) == 1
     assert lib.jtmoe_moe_forward_takes_decode_path(16, H, E, K, I, bf) == 1   # T * K = 2 * E
