@@ -271,11 +271,10 @@ int jtmoe_smebu_update(const float* router_counts, float* momentum, float* exper
  *        which needs nothing of the routing -- while a few of its workgroups are the
  *        router and write the dispatch plan; the down launch then takes the routed rows.
  *        The workspace then holds the activations [E,T,I]; results are bit for bit those
- *        of the other path.  That launch counts its router workgroups in one of 64 words
- *        of device memory inside the library (zero at load, set back to zero by the
- *        launch); the host hands the words out round-robin, so more than 64 such calls
- *        in flight at once on one GPU are not supported.  No counterpart in the
- *        reference (XLA decides its own fusions).
+ *        of the other path.  That launch counts its router workgroups in a word of the
+ *        workspace (tagged per launch, so the workspace needs no clearing): like every
+ *        call, it shares no state with calls that use other workspaces.  No counterpart
+ *        in the reference (XLA decides its own fusions).
  */
 int jtmoe_moe_forward_takes_decode_path(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int dtype);
 size_t jtmoe_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t K, int64_t I, int64_t Is, int dtype);

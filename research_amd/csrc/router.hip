@@ -15,6 +15,8 @@
 #include "grouped_gemm_dma.hpp"
 
 #include <atomic>
+#include <chrono>
+#include <random>
 
 #include <mutex>
 
@@ -72,6 +74,9 @@ __host__ __device__ inline RouterScratch router_scratch(void* ws, int E) {
 }
 
 inline size_t router_scratch_bytes(int64_t E) { return align_up((size_t)E * 12, 256); }
+// the partial sums of the small-batch kernels start behind the scratch; the arrival word of the decode
+// launch behind them
+inline size_t router_arrivals_offset(int64_t E);
 
 __global__ void router_zero_kernel(void* ws, int E) {
   RouterScratch s = router_scratch(ws, E);
@@ -801,6 +806,10 @@ __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
                                   counts, importance, group_sizes, offsets, source_order, inverse, score_func);
 }
 
+inline size_t router_arrivals_offset(int64_t E) {
+  return router_scratch_bytes(E) + align_up((size_t)kPartialMaxSlices * kSplitMaxTokens * E * sizeof(float), 256);
+}
+
 // ---------------------------------------------------------------------------
 // The decode launch: ONE launch in which most workgroups stream the gate and up matrices (every token
 // through every expert, grouped_gemm_dma_tile in its uniform mode -- nothing of that needs the routing)
@@ -810,14 +819,27 @@ __global__ __launch_bounds__(4 * kTok) void router_finish_kernel(
 // in the same order as the two-launch form, so the same bits.  The router's 21 us of dependent steps
 // then run beside the 115 us of weight streaming instead of in front of it, with no second stream and
 // no dependency between launches other than the stream's own order.
-// The arrival counter of a launch is one of kDecodeSlots words of device memory that are zero when the
-// library is loaded; the last workgroup to arrive sets its word back to zero.  The host hands the slots
-// out round-robin, so launches that overlap on one GPU (from several streams) use different words unless
-// more than kDecodeSlots of them are in flight at once.
+// The arrival counter is a 64-bit word of the caller's workspace: the low byte counts, the rest is a tag
+// the host draws per launch.  A word whose tag is not this launch's counts as zero, so the word needs no
+// clearing before its first use (the workspace arrives with whatever it held; the first tag of a process
+// is random, 56 bits); the workgroup that finishes writes zero, so a captured launch, whose tag is the
+// same at every replay, starts from zero as well.  No state outside the workspace: calls are as
+// re-entrant as their workspaces are distinct.
 // ---------------------------------------------------------------------------
-constexpr int kDecodeSlots = 64;
-__device__ unsigned g_decode_arrivals[kDecodeSlots];
-std::atomic<unsigned> g_decode_next_slot{0};
+std::atomic<unsigned long long> g_decode_tag{0};
+
+unsigned long long next_decode_tag() {
+  unsigned long long t = g_decode_tag.load(std::memory_order_relaxed);
+  if (t == 0) {  // first use in this process
+    std::random_device rd;
+    unsigned long long seed = ((unsigned long long)rd() << 32) ^ rd() ^
+                              (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count();
+    unsigned long long expected = 0;
+    g_decode_tag.compare_exchange_strong(expected, seed | 1ull, std::memory_order_relaxed);
+  }
+  t = g_decode_tag.fetch_add(1ull, std::memory_order_relaxed) & 0x00ffffffffffffffull;
+  return (t == 0 ? 1ull : t) << 8;
+}
 
 template <int NB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void decode_gate_up_router_kernel(
@@ -827,7 +849,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void d
     int32_t* __restrict__ ids, bf16_raw* __restrict__ weights, float* __restrict__ scores,
     float* __restrict__ counts, float* __restrict__ importance, int32_t* __restrict__ group_sizes,
     int32_t* __restrict__ offsets, int32_t* __restrict__ source_order, int32_t* __restrict__ inverse,
-    float* __restrict__ partial, int token_blocks, int slices, int slot) {
+    float* __restrict__ partial, int token_blocks, int slices, unsigned long long* __restrict__ arrivals,
+    unsigned long long tag) {
   constexpr int E = NB * 16;
   const int router_blocks = token_blocks * slices;
   if ((int)blockIdx.x >= router_blocks) {
@@ -850,14 +873,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void d
   __syncthreads();
   if (threadIdx.x == 0) {
     __threadfence();
-    is_last = atomicAdd(&g_decode_arrivals[slot], 1u) == (unsigned)(router_blocks - 1);
+    unsigned long long seen = atomicAdd(arrivals, 0ull), assumed;
+    unsigned count;
+    do {  // lock-free: some workgroup's exchange always succeeds
+      assumed = seen;
+      count = (assumed >> 8) == (tag >> 8) ? (unsigned)(assumed & 0xffull) : 0u;
+      seen = atomicCAS(arrivals, assumed, tag | (unsigned long long)(count + 1u));
+    } while (seen != assumed);
+    is_last = count + 1u == (unsigned)router_blocks;
     if (is_last) __threadfence();
   }
   __syncthreads();
   if (!is_last) return;
   router_finish_body<64, true>(partial, slices, bias, T, E, K, route_scale, ids, weights, scores, nullptr, counts,
                                importance, group_sizes, offsets, source_order, inverse, score_func);
-  if (threadIdx.x == 0) g_decode_arrivals[slot] = 0u;
+  if (threadIdx.x == 0) *arrivals = 0ull;
 }
 
 template <typename KernelT>
@@ -1070,7 +1100,10 @@ int launch_decode_gate_up_router(const void* x, const void* w_router, const floa
   const int64_t mtiles = E * ((T + GateUpTinyCfg::BM - 1) / GateUpTinyCfg::BM);
   const int64_t nt = (I + GateUpTinyCfg::BN - 1) / GateUpTinyCfg::BN;
   const int64_t grid = (int64_t)token_blocks * slices + gemm_grid(mtiles, nt);
-  const int slot = (int)(g_decode_next_slot.fetch_add(1u, std::memory_order_relaxed) % kDecodeSlots);
+  if (token_blocks * slices > 255) return fail(JTMOE_EUNSUPPORTED, "moe_forward: decode launch with %d router workgroups", token_blocks * slices);
+  unsigned long long* const arrivals = reinterpret_cast<unsigned long long*>(
+      static_cast<unsigned char*>(router_workspace) + router_arrivals_offset(E));
+  const unsigned long long tag = next_decode_tag();
 #define JT_DECODE_CASE(NB)                                                                                       \
   case NB * 16: {                                                                                                \
     auto kernel = decode_gate_up_router_kernel<NB>;                                                              \
@@ -1081,7 +1114,7 @@ int launch_decode_gate_up_router(const void* x, const void* w_router, const floa
         static_cast<uint16_t*>(act_full), (int)T, (int)H, (int)I, (int)mtiles, (int)nt,                          \
         static_cast<const uint16_t*>(w_router), expert_bias, (int)K, (float)route_scale, score_func, expert_ids, \
         static_cast<bf16_raw*>(weights), scores, expert_counts, importance, group_sizes, offsets, source_order,  \
-        inverse, partial, token_blocks, slices, slot);                                                           \
+        inverse, partial, token_blocks, slices, arrivals, tag);                                                  \
   } break;
   switch ((int)E) {
     JT_DECODE_CASE(1)
@@ -1125,8 +1158,8 @@ using namespace jtmoe;
 
 extern "C" size_t jtmoe_router_workspace_bytes(int64_t E) {
   if (E <= 0) return 0;
-  // the statistics accumulators, then the partial sums of the small-batch path
-  return router_scratch_bytes(E) + align_up((size_t)kPartialMaxSlices * kSplitMaxTokens * E * sizeof(float), 256);
+  // the statistics accumulators, the partial sums of the small-batch path, the arrival word of the decode launch
+  return router_arrivals_offset(E) + 256;
 }
 
 extern "C" int jtmoe_router(const void* x, const void* w_router, const float* expert_bias, int64_t T, int64_t H,

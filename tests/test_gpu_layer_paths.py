@@ -197,3 +197,33 @@ def test_decode_path_follows_work_on_the_callers_stream(gpu):
             del filler
     torch.cuda.current_stream(gpu).wait_stream(stream)
     torch.cuda.synchronize()
+
+
+def test_decode_path_on_two_streams_at_once(gpu):
+    """Calls share no state but their arguments: decode calls enqueued on two streams, each with its own
+    workspace and outputs, may run at the same time and give the results of calls made one after the other
+    (the arrival word of the decode launch lives in the workspace; also after a workspace was filled with
+    ones, i.e. starts from a word that is neither zero nor a tag)."""
+    rng = np.random.default_rng(5)
+    T, H, E, K, I = 64, 1024, 64, 8, 256
+    w_router = dev((rng.standard_normal((H, E)) * 0.1).astype(np.float32), gpu, "bf16")
+    gate = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    up = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    down = dev((rng.standard_normal((E, I, H)) * 0.05).astype(np.float32), gpu, "bf16")
+    xs = [dev(rng.standard_normal((T, H)).astype(np.float32), gpu, "bf16") for _ in range(2)]
+    want = [ops.moe_forward(x, w_router, None, gate, up, down, K, 1.0) for x in xs]
+    torch.cuda.synchronize()
+    nbytes = ops._lib().jtmoe_workspace_bytes(T, H, E, K, I, 0, ops._code(torch.bfloat16))
+    spaces = [torch.full((nbytes,), 0xff, dtype=torch.uint8, device=gpu) for _ in range(2)]
+    streams = [torch.cuda.Stream(device=gpu) for _ in range(2)]
+    torch.cuda.synchronize()  # the fills above ran on the default stream
+    got = [[], []]
+    for _ in range(20):
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                got[i].append(ops.moe_forward(xs[i], w_router, None, gate, up, down, K, 1.0, workspace=spaces[i]))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for r in got[i]:
+            assert torch.equal(r.y, want[i].y) and torch.equal(r.source_order, want[i].source_order)
+            assert torch.equal(r.expert_counts, want[i].expert_counts)
