@@ -227,3 +227,34 @@ def test_decode_path_on_two_streams_at_once(gpu):
         for r in got[i]:
             assert torch.equal(r.y, want[i].y) and torch.equal(r.source_order, want[i].source_order)
             assert torch.equal(r.expert_counts, want[i].expert_counts)
+
+
+@pytest.mark.parametrize("tokens", [40, 64, 300, 3000])
+def test_layer_statistics_with_a_non_finite_token(gpu, tokens):
+    """A token whose input is NaN has NaN logits, scores and route weights.  Its ids stay inside [0, E)
+    (NaN scores are chosen last, lower index first: experts 0 .. K-1), it is counted like any other token,
+    and its NaN weights add nothing to the importance sums (a 32.32 fixed-point sum has no NaN) -- on every
+    route the statistics take: the router's finishing workgroup, the decode launch, the one-workgroup
+    dispatch and the histogram pass."""
+    rng = np.random.default_rng(tokens)
+    H, E, K, I = 256, 64, 8, 64
+    x = rng.standard_normal((tokens, H)).astype(np.float32)
+    x[3, :] = np.nan
+    w_router = dev((rng.standard_normal((H, E)) * 0.1).astype(np.float32), gpu, "bf16")
+    gate = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    up = dev((rng.standard_normal((E, H, I)) * 0.05).astype(np.float32), gpu, "bf16")
+    down = dev((rng.standard_normal((E, I, H)) * 0.05).astype(np.float32), gpu, "bf16")
+    layer = ops.moe_forward(dev(x, gpu, "bf16"), w_router, None, gate, up, down, K, 1.0)
+    ids, weights = host(layer.expert_ids), host(layer.weights)
+    assert ids.min() >= 0 and ids.max() < E
+    assert ids[3].tolist() == list(range(K)) and np.all(np.isnan(weights[3]))
+    assert np.array_equal(host(layer.expert_counts), np.bincount(ids.reshape(-1), minlength=E).astype(np.float32))
+    importance = host(layer.importance)
+    assert np.all(np.isfinite(importance))
+    clean = np.where(np.isnan(weights), 0.0, weights).astype(np.float64)
+    want = np.zeros(E)
+    np.add.at(want, ids.reshape(-1), clean.reshape(-1))
+    np.testing.assert_allclose(importance, want, rtol=1e-5, atol=1e-5)
+    # every other token is untouched by its neighbour
+    others = np.delete(np.arange(tokens), 3)
+    assert np.all(np.isfinite(host(layer.y)[others]))
