@@ -852,6 +852,14 @@ int main(int argc, char** argv) {
           timeit_cold<GateUpStreamCfg>(name, g2, 20);
         }
       g_chunk = -1;
+      // the same launch with 64-deep steps in two stages, and with the older kernel
+      for (int rep = 0; rep < 3; ++rep) {
+        g_stream = true;
+        timeit_cold<GateUpStreamCfg>("C2 gate/up stream 4 x 32 (library)", g2, 20);
+        timeit_cold<GateUpStream2Cfg>("C2 gate/up stream 2 x 64", g2, 20);
+        g_stream = false;
+        timeit_cold<GateUpCfg>("C2 gate/up, older kernel", g2, 20);
+      }
       g_stream = false;
       release(g2);
     }
