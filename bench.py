@@ -115,7 +115,7 @@ def cpu_baseline(name: str, sample_tokens: int | None) -> dict:
     )
 
 
-def graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps) -> dict:
+def graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, warmup=3) -> dict:
     """Small batches are bound by launching the layer's kernels from Python, not by the kernels: the same
     calls captured once into a HIP graph and replayed."""
     import torch
@@ -123,7 +123,7 @@ def graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps) -> dict:
     from research_amd.graph import GraphedLayer
 
     layer = GraphedLayer(x, w_r, bias, gate, upw, down, cfg["K"], 1.0, shared=shared)
-    for _ in range(3):
+    for _ in range(max(warmup, 3)):
         layer.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -134,7 +134,7 @@ def graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps) -> dict:
     return {"ms_per_step": ms, "tokens_per_s": x.shape[0] / (ms * 1e-3), "steps": steps}
 
 
-def block_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, layer_ms) -> dict:
+def block_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, layer_ms, warmup=3) -> dict:
     """x + post_norm(moe(pre_norm(x))): the layer with the decoder block's two RMSNorms and the residual
     add around it (the post-norm and the add run inside the combine kernel)."""
     import torch
@@ -148,7 +148,7 @@ def block_timing(x, w_r, bias, gate, upw, down, shared, cfg, steps, layer_ms) ->
     def step():
         return ops.ffn_block_forward(x, pre, post, 1e-6, w_r, bias, gate, upw, down, cfg["K"], 1.0, shared=shared)
 
-    for _ in range(3):
+    for _ in range(max(warmup, 3)):  # as many as the layer's own timing gets: the legs before this one let the clocks drop
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -432,8 +432,8 @@ def main() -> int:
                                   "expert and holds the router and the dispatch plan in a few of its workgroups")
     if not args.no_block:
         if T <= 2048:
-            line["graph_replay"] = graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, max(args.steps, 50))
-        line["block"] = block_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, ms_per_step)
+            line["graph_replay"] = graph_timing(x, w_r, bias, gate, upw, down, shared, cfg, max(args.steps, 50), args.warmup)
+        line["block"] = block_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, ms_per_step, args.warmup)
     if not args.no_train:
         line["train"] = train_timing(x, w_r, bias, gate, upw, down, shared, cfg, args.steps, work)
     if not args.no_cpu_baseline:
