@@ -108,9 +108,10 @@ def route_weight_grad_rounded(x, expert_ids, gate, up, down, dy, rounded=True):
     h = silu(g) u, g = x[t] Wg[e], u = x[t] Wu[e] (the same number: both are dy^T Wd^T h), where a
     bf16 implementation rounds g, u, h and Z to bf16 before the inner product and the result after it.
 
-    Returns (value, budget), both [T,K].  budget[t,s] = 2^-9 * (sum_i |Z_i h_i| (3 + kappa_i) + |value|)
+    Returns (value, budget), both [T,K].  budget[t,s] = 2^-8 * (sum_i |Z_i h_i| (3 + kappa_i) + |value|)
     with kappa = |d ln silu(g) / d ln g| = |1 + g (1 - sigmoid(g))|: the first-order bound on
-    |value - exact| from one relative rounding of 2^-9 on each of Z, u, h (factor 1 each) and g
+    |value - exact| from one relative rounding of at most 2^-8 (the unit roundoff of bf16: half a
+    unit in the last of its 8 significant bits) on each of Z, u, h (factor 1 each) and g
     (factor kappa), plus the rounding of the result.  With cancellation in the sum the exact value can
     be far smaller than sum_i |Z_i h_i|, which is why a bound relative to the value itself (or, for a
     tensor of one element, to the tensor's maximum) does not hold for this quantity.
@@ -130,7 +131,7 @@ def route_weight_grad_rounded(x, expert_ids, gate, up, down, dy, rounded=True):
         z = rnd(dy[t_idx] @ down[e].T)
         value[t_idx, s_idx] = rnd(np.sum(z * h, axis=-1))
         kappa = np.abs(1.0 + g * (1.0 - sig))
-        budget[t_idx, s_idx] = 2.0**-9 * (np.sum(np.abs(z * h) * (3.0 + kappa), axis=-1) + np.abs(value[t_idx, s_idx]))
+        budget[t_idx, s_idx] = 2.0**-8 * (np.sum(np.abs(z * h) * (3.0 + kappa), axis=-1) + np.abs(value[t_idx, s_idx]))
     return value, budget
 
 

@@ -92,6 +92,9 @@ def test_expert_gradients_match_oracle(gpu, tokens, hidden, experts, top_k, inte
         print(f"[parity] {tag} d_weights: max err/budget = {float(np.max(np.abs(dw - want.d_weights) / budget)):.3f}; "
               f"against the rounded evaluation: {float(np.max(np.abs(dw - value) / budget)):.3f}", flush=True)
         assert np.all(np.abs(dw - want.d_weights) <= budget)
+        # and the kernel's own value to the same evaluation with the same roundings made in float64: what is
+        # left between the two is a factor that the kernel's fp32 sums rounded the other way
+        assert np.all(np.abs(dw - value) <= 0.5 * budget)
     else:
         np.testing.assert_allclose(host(res.gate_pre), ref_g, rtol=2e-5, atol=2e-5)
         np.testing.assert_allclose(host(res.up_pre), ref_u, rtol=2e-5, atol=2e-5)

@@ -202,7 +202,19 @@ def test_route_weight_grad_without_rounding_is_the_exact_gradient():
     np.testing.assert_allclose(value, exact, rtol=1e-12, atol=1e-14)
 
 
-@pytest.mark.parametrize("shape", SINGLE_TOKEN_SHAPES + [(300, 64, 6, 3, 96), (40, 200, 5, 2, 136)])
+def test_unit_roundoff_of_bf16_is_two_to_the_minus_eight():
+    """What the budget multiplies: rounding to bf16 (8 significant bits, nearest even) moves a value by at
+    most 2^-8 of itself, and by nearly that much just above a power of two -- half of it would not be a
+    bound (an element with few terms can exceed a budget built on 2^-9)."""
+    a = np.linspace(1.0, 2.0, 100001)
+    rel = np.abs(G._bf16(a) - a) / a
+    assert rel.max() <= 2.0**-8
+    worst = 1.0 + 2.0**-8 * 0.999  # just under the midpoint of 1 and 1 + 2^-7: rounds down to 1
+    assert G._bf16(np.array([worst]))[0] == 1.0 and (worst - 1.0) / worst > 0.99 * 2.0**-8
+
+
+@pytest.mark.parametrize("shape", SINGLE_TOKEN_SHAPES + [(300, 64, 6, 3, 96), (40, 200, 5, 2, 136), (300, 200, 5, 3, 8),
+                                                         (300, 64, 5, 4, 8)])
 def test_bf16_rounding_explains_the_route_weight_gradient_error(shape):
     """The four bf16 roundings in front of <Z, h> move the result by no more than their first-order
     budget, and that budget, not the size of the exact value, is what a bf16 result can be held to."""
@@ -217,10 +229,10 @@ def test_bf16_rounding_explains_the_route_weight_gradient_error(shape):
 def test_single_token_error_is_the_one_seen_on_the_gpu():
     """(1, 8, 1, 1, 256): exact 0.2014, rounded 0.1943 -- 3.515e-2 of the exact value, the figure a bf16
     backward pass on the GPU printed for this shape; (1, 8, 16, 1, 136): the terms cancel to -1.7e-4 and
-    the same roundings leave -5.8e-3, 33 times the exact value.  Both are under a quarter of the budget."""
+    the same roundings leave -5.8e-3, 33 times the exact value.  Both are under an eighth of the budget."""
     for shape, rel in (((1, 8, 1, 1, 256), 3.515e-2), ((1, 8, 16, 1, 136), 3.327e1)):
         x, gate, up, down, ids, w, dy = single_token_problem(*shape)
         exact = G.experts_backward(x, ids, w, gate, up, down, dy).d_weights
         value, budget = G.route_weight_grad_rounded(x, ids, gate, up, down, dy)
         assert abs(np.abs(value - exact).max() / np.abs(exact).max() - rel) <= 1e-3 * rel
-        assert np.all(np.abs(value - exact) <= 0.25 * budget)
+        assert np.all(np.abs(value - exact) <= 0.125 * budget)
