@@ -16,7 +16,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
-from research_amd import ops
+from research_amd import _ffi, ops
 from test_gpu_parity import dev, host
 
 pytestmark = pytest.mark.gpu
@@ -171,6 +171,29 @@ def test_decode_path_equals_the_stand_alone_operators(gpu, tokens, hidden, exper
     again = ops.moe_forward(x, w_router, None, gate, up, down, top_k, 1.0, shared=shared)
     assert torch.equal(again.y, want)
     torch.cuda.synchronize()
+
+
+def test_decode_path_on_seeded_random_shapes(gpu):
+    """The same comparison on 48 shapes drawn around the path's conditions (token counts either side of 64
+    and of top_k * tokens = 2 * experts, 8 ... 64 experts, hidden sizes with one, several and ragged
+    slices, with and without shared experts): whichever path a shape takes, the layer equals its operators
+    called one by one."""
+    rng = np.random.default_rng(20251)
+    taken = 0
+    for _ in range(48):
+        experts = int(rng.choice([8, 16, 32, 64]))
+        top_k = int(rng.integers(1, min(experts, 16) + 1))
+        tokens = int(rng.integers(1, 70))
+        hidden = int(rng.choice([128, 192, 256, 384, 512, 640, 1024, 1152, 2048, 2176]))
+        d_ff = int(rng.choice([64, 128, 192, 320, 704]))
+        shared_width = int(rng.choice([0, 0, 64, 128]))
+        decode = bool(_ffi.load_library().jtmoe_moe_forward_takes_decode_path(tokens, hidden, experts, top_k, d_ff,
+                                                                             _ffi.JTMOE_BF16))
+        taken += decode
+        print(f"[layer paths] decode sweep: T={tokens} H={hidden} E={experts} K={top_k} I={d_ff} shared={shared_width} "
+              f"decode path={decode}", flush=True)
+        test_decode_path_equals_the_stand_alone_operators(gpu, tokens, hidden, experts, top_k, d_ff, shared_width)
+    assert 8 <= taken <= 40  # the draw covers both sides
 
 
 def test_decode_path_follows_work_on_the_callers_stream(gpu):
