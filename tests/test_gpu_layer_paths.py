@@ -252,6 +252,54 @@ def test_decode_path_on_two_streams_at_once(gpu):
             assert torch.equal(r.expert_counts, want[i].expert_counts)
 
 
+def test_calls_from_four_host_threads_at_once(gpu):
+    """The entry points are called from whatever thread the host's executor uses
+    (src/jaxtitan/kernels/cuda/rmsnorm/rmsnorm_ffi.cu:59-68: re-entrant, work only on the stream handed in):
+    four threads, each with its own stream, workspace and shape -- a decode call, a small batch, one that
+    takes the large-batch kernels, one in fp32 -- call the layer 25 times each at the same time (ctypes
+    releases the interpreter lock for the duration of a call) and get what a single thread got."""
+    import threading
+
+    rng = np.random.default_rng(9)
+    cases = []
+    for tokens, hidden, experts, top_k, d_ff, dtype in [(64, 512, 64, 8, 128, "bf16"), (200, 256, 16, 2, 192, "bf16"),
+                                                        (1500, 512, 32, 4, 128, "bf16"), (90, 64, 8, 2, 40, "f32")]:
+        a = [dev(rng.standard_normal((tokens, hidden)).astype(np.float32), gpu, dtype),
+             dev((rng.standard_normal((hidden, experts)) * 0.1).astype(np.float32), gpu, dtype), None,
+             dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, dtype),
+             dev((rng.standard_normal((experts, hidden, d_ff)) * 0.05).astype(np.float32), gpu, dtype),
+             dev((rng.standard_normal((experts, d_ff, hidden)) * 0.05).astype(np.float32), gpu, dtype), top_k, 1.0]
+        cases.append((a, ops.moe_forward(*a)))
+    torch.cuda.synchronize()
+    errors: list[str] = []
+    start = threading.Barrier(len(cases))
+
+    def worker(i):
+        args, want = cases[i]
+        try:
+            stream = torch.cuda.Stream(device=gpu)
+            start.wait()
+            with torch.cuda.stream(stream):
+                for n in range(25):
+                    got = ops.moe_forward(*args)
+                    stream.synchronize()
+                    for name in ("y", "expert_ids", "weights", "scores", "expert_counts", "importance", "source_order"):
+                        if not torch.equal(getattr(got, name), getattr(want, name)):
+                            errors.append(f"thread {i} call {n}: {name} differs")
+                            return
+        except Exception as exc:  # noqa: BLE001 -- reported by the assertion below
+            errors.append(f"thread {i}: {type(exc).__name__}: {exc}")
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(cases))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    torch.cuda.synchronize()
+    assert not any(t.is_alive() for t in threads), "a thread did not finish"
+    assert not errors, errors[:4]
+
+
 @pytest.mark.parametrize("tokens", [40, 64, 300, 3000])
 def test_layer_statistics_with_a_non_finite_token(gpu, tokens):
     """A token whose input is NaN has NaN logits, scores and route weights.  Its ids stay inside [0, E)
