@@ -153,3 +153,33 @@ def test_graph_replay_matches_eager_on_every_replay(gpu):
         assert torch.equal(got.expert_ids, eager.expert_ids) and torch.equal(got.weights, eager.weights)
         assert torch.equal(got.expert_counts, eager.expert_counts) and torch.equal(got.inverse, eager.inverse)
         (eager.y.float() * 2).sum().item()  # unrelated eager work between the replays
+
+
+@pytest.mark.parametrize("tokens,hidden,experts,top_k,d_ff,shared_width",
+                         [(600, 512, 16, 2, 256, 128),   # router, histogram, rank, four GEMMs, combine
+                          (200, 256, 64, 8, 64, 0),      # the small-batch router with the plan in its last workgroup
+                          (3000, 1024, 128, 8, 128, 0)])  # many short groups
+def test_graph_replay_of_the_other_layer_paths(gpu, tokens, hidden, experts, top_k, d_ff, shared_width):
+    """The same for the launches a call makes outside the decode path: every replay, with eager work and
+    synchronisations between them, gives what the eager call gives on the same input."""
+    from research_amd import ops
+    from research_amd.graph import GraphedLayer
+
+    gen = torch.Generator(device=gpu).manual_seed(tokens)
+    draw = lambda *shape, std=1.0: (torch.randn(*shape, device=gpu, generator=gen) * std).to(torch.bfloat16)
+    params = (draw(hidden, experts, std=0.1), None, draw(experts, hidden, d_ff, std=0.05),
+              draw(experts, hidden, d_ff, std=0.05), draw(experts, d_ff, hidden, std=0.05))
+    shared = None
+    if shared_width:
+        shared = (draw(hidden, shared_width, std=0.05), draw(hidden, shared_width, std=0.05),
+                  draw(shared_width, hidden, std=0.05))
+    layer = GraphedLayer(draw(tokens, hidden), *params, top_k, 1.0, shared=shared)
+    for i in range(4):
+        x = draw(tokens, hidden)
+        eager = ops.moe_forward(x, *params, top_k, 1.0, shared=shared)
+        torch.cuda.synchronize()
+        got = layer.replay(x)
+        torch.cuda.synchronize()
+        for name in ("y", "expert_ids", "weights", "scores", "expert_counts", "importance", "group_sizes", "inverse"):
+            assert torch.equal(getattr(got, name), getattr(eager, name)), f"replay {i}: {name}"
+        (eager.y.float() * 2).sum().item()  # unrelated eager work between the replays
