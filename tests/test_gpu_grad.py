@@ -349,3 +349,45 @@ def test_sequence_balance_loss_gradient_matches_oracle(gpu, batch, seq, experts,
     assert float(loss.detach()) == pytest.approx(float(O.sequence_balance_loss(ids, scores, top_k)), rel=1e-5)
     (g,) = torch.autograd.grad(loss * 0.25, [s_req])
     np.testing.assert_allclose(host(g) / scale, 0.25 * want / scale, rtol=1e-4, atol=2e-6)
+
+
+def test_training_step_replays_from_a_captured_graph(gpu):
+    """Forward with residuals and the backward pass only enqueue kernels, so a training step can be captured
+    once and replayed (the reference's step runs inside one compiled program, steps/train_step.py): every
+    replay, with eager work and synchronisations between them, gives the eager call's gradients bit for bit."""
+    tokens, hidden, experts, top_k, inter, shared_inter = 700, 256, 16, 2, 192, 128
+    gen = torch.Generator(device=gpu).manual_seed(21)
+    draw = lambda *shape, std=1.0: (torch.randn(*shape, device=gpu, generator=gen) * std).to(torch.bfloat16)
+    w_router, gate, up = draw(hidden, experts, std=0.1), draw(experts, hidden, inter, std=0.05), draw(experts, hidden, inter, std=0.05)
+    down = draw(experts, inter, hidden, std=0.05)
+    shared = (draw(hidden, shared_inter, std=0.05), draw(hidden, shared_inter, std=0.05), draw(shared_inter, hidden, std=0.05))
+
+    def step(x, dy):
+        result, residuals = grad.moe_forward_train(x, w_router, None, gate, up, down, top_k, 1.0, shared=shared)
+        return result, grad.moe_backward(x, dy, None, w_router, gate, up, down, shared, result, residuals, 1.0)
+
+    x_in, dy_in = draw(tokens, hidden), draw(tokens, hidden)
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream(gpu))
+    with torch.cuda.stream(side):
+        for _ in range(2):  # first calls set kernel attributes and size the workspaces
+            step(x_in, dy_in)
+    torch.cuda.current_stream(gpu).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured_result, captured = step(x_in, dy_in)
+    for i in range(4):
+        x, dy = draw(tokens, hidden), draw(tokens, hidden)
+        eager_result, eager = step(x, dy)
+        torch.cuda.synchronize()
+        x_in.copy_(x)
+        dy_in.copy_(dy)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured_result.y, eager_result.y), f"replay {i}: y"
+        for name in ("dx", "d_w_router", "d_gate", "d_up", "d_down"):
+            assert torch.equal(getattr(captured, name), getattr(eager, name)), f"replay {i}: {name}"
+        for a, b in zip(captured.d_shared, eager.d_shared):
+            assert torch.equal(a, b), f"replay {i}: shared gradient"
+        (eager.dx.float() * 2).sum().item()  # unrelated eager work between the replays
