@@ -98,7 +98,6 @@ __global__ void router_finalize_kernel(const void* ws, int E, float* counts, flo
 struct RouterSmem {
   float* tile;       // [kRouterTokens][E+1] logits, then scores
   float* bias;       // [E]
-  float* top_score;  // [kRouterTokens][K]
   int* top_id;       // [kRouterTokens][K]
   int* cnt;          // [E]
   unsigned long long* imp;  // [E]
@@ -109,7 +108,7 @@ __host__ __device__ inline size_t router_smem_bytes(int E, int K, int kRouterTok
   n += (size_t)E * 8;                        // imp (first: 8-byte aligned)
   n += (size_t)kRouterTokens * (E + 1) * 4;  // tile
   n += (size_t)E * 4;                        // bias
-  n += (size_t)kRouterTokens * K * 4 * 2;    // top_score, top_id
+  n += (size_t)kRouterTokens * K * 4;        // top_id
   n += (size_t)E * 4;                        // cnt
   return n;
 }
@@ -119,8 +118,7 @@ __device__ __forceinline__ RouterSmem router_smem(unsigned char* base, int E, in
   s.imp = reinterpret_cast<unsigned long long*>(base);
   s.tile = reinterpret_cast<float*>(s.imp + E);
   s.bias = s.tile + kRouterTokens * (E + 1);
-  s.top_score = s.bias + E;
-  s.top_id = reinterpret_cast<int*>(s.top_score + kRouterTokens * K);
+  s.top_id = reinterpret_cast<int*>(s.bias + E);
   s.cnt = s.top_id + kRouterTokens * K;
   return s;
 }
@@ -152,8 +150,21 @@ __device__ __forceinline__ int order_key(float v) {
 
 // K rounds of "largest remaining score + bias, lower index on ties" for one token, by its four
 // lanes: lane q owns experts [e_begin, e_begin + EQ) and keeps their keys in registers; a taken
-// expert's key becomes kTakenKey, below every real value, so a round is one compare and two
-// selects per expert.
+// expert's key becomes kTakenKey, below every real value.  A round: the largest key of the token (a run
+// of max operations in the lane, two exchanges inside the quad), the lowest index that holds it (the
+// lane's own, scanned downwards so that the lowest wins, then the minimum over the quad), and the key at
+// that index retired -- no branch, and nothing that waits for the LDS.
+constexpr int kNoExpert = 0x7fffffff;
+template <int kXor>
+__device__ __forceinline__ int quad_max_i32(int v) {
+  const int o = quad_xor_i32<kXor>(v);
+  return o > v ? o : v;
+}
+template <int kXor>
+__device__ __forceinline__ int quad_min_i32(int v) {
+  const int o = quad_xor_i32<kXor>(v);
+  return o < v ? o : v;
+}
 template <int EQ>
 __device__ __forceinline__ void select_from_registers(const RouterSmem& sm, const float* row, int e_begin, bool row_ok,
                                                       int t, int q, int K) {
@@ -162,38 +173,20 @@ __device__ __forceinline__ void select_from_registers(const RouterSmem& sm, cons
 #pragma unroll
   for (int j = 0; j < EQ; ++j) key[j] = row_ok ? order_key(row[e_begin + j] + sm.bias[e_begin + j]) : kTakenKey;
   for (int r = 0; r < K; ++r) {
-    int best_k = kTakenKey, best_e = -1;
+    int best_k = key[0];
 #pragma unroll
-    for (int j = 0; j < EQ; ++j) {
-      const bool better = key[j] > best_k;  // strictly: the lower index keeps a tie
-      best_k = better ? key[j] : best_k;
-      best_e = better ? e_begin + j : best_e;
-    }
-    {
-      const int ok = quad_xor_i32<1>(best_k);
-      const int oe = quad_xor_i32<1>(best_e);
-      if (oe >= 0 && (best_e < 0 || ok > best_k || (ok == best_k && oe < best_e))) {
-        best_k = ok;
-        best_e = oe;
-      }
-    }
-    {
-      const int ok = quad_xor_i32<2>(best_k);
-      const int oe = quad_xor_i32<2>(best_e);
-      if (oe >= 0 && (best_e < 0 || ok > best_k || (ok == best_k && oe < best_e))) {
-        best_k = ok;
-        best_e = oe;
-      }
-    }
-    if (row_ok) {
-      const int own = best_e - e_begin;
+    for (int j = 1; j < EQ; ++j) best_k = key[j] > best_k ? key[j] : best_k;
+    best_k = quad_max_i32<1>(best_k);
+    best_k = quad_max_i32<2>(best_k);
+    int best_e = kNoExpert;
 #pragma unroll
-      for (int j = 0; j < EQ; ++j) key[j] = j == own ? kTakenKey : key[j];
-      if (q == 0) {
-        sm.top_id[t * K + r] = best_e;
-        sm.top_score[t * K + r] = row[best_e];
-      }
-    }
+    for (int j = EQ - 1; j >= 0; --j) best_e = key[j] == best_k ? e_begin + j : best_e;
+    best_e = quad_min_i32<1>(best_e);
+    best_e = quad_min_i32<2>(best_e);
+    const int own = best_e - e_begin;
+#pragma unroll
+    for (int j = 0; j < EQ; ++j) key[j] = j == own ? kTakenKey : key[j];
+    if (row_ok && q == 0) sm.top_id[t * K + r] = best_e;
   }
 }
 
@@ -230,10 +223,7 @@ __device__ __forceinline__ void select_from_lds(const RouterSmem& sm, const floa
     if (row_ok) {
       const int j = best_e - e_begin;
       if (j >= 0 && j < eq) taken |= 1ull << j;
-      if (q == 0) {
-        sm.top_id[t * K + r] = best_e;
-        sm.top_score[t * K + r] = row[best_e];
-      }
+      if (q == 0) sm.top_id[t * K + r] = best_e;
     }
   }
 }
@@ -330,12 +320,12 @@ __device__ void router_epilogue(const RouterSmem& sm, const float* __restrict__ 
   // renormalise: the lanes of a token share out its K slots; each adds up the denominator itself, in
   // slot order
   if (row_ok) {
-    float denom = sm.top_score[t * K];
-    for (int r = 1; r < K; ++r) denom = denom + sm.top_score[t * K + r];
+    float denom = row[sm.top_id[t * K]];
+    for (int r = 1; r < K; ++r) denom = denom + row[sm.top_id[t * K + r]];
     denom = denom + 1e-20f;
     for (int r = q; r < K; r += 4) {
       const int e = sm.top_id[t * K + r];
-      float w = sm.top_score[t * K + r] / denom;
+      float w = row[e] / denom;
       w = w * route_scale;
       w = Elem<T>::round(w);
       const size_t o = (size_t)(t0 + t) * K + r;
